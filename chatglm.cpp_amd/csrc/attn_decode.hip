@@ -2,148 +2,126 @@
 //
 // One launch does rope(q, k), the K/V append and the attention of one layer (chatglm.cpp:655-717 for
 // qlen == 1).  The cache sequence of each KV group is cut into 64-key tiles that are dealt out to
-// nsplit workgroups x `waves` wavefronts; every wave issues the loads of a whole tile (16 KiB of K
-// rows and 16 KiB of V columns) before it does anything else, so that a full grid keeps the whole
-// layer's cache in flight at once.  The up to 16 query heads of the group are the 16 columns of
-// v_mfma_f32_16x16x32_f16 tiles: S^T = K q^T puts keys on the rows, which is exactly the layout the
-// second product O^T = V^T P^T wants for P^T, so probabilities go from accumulator registers to
-// operand registers without touching LDS.  Waves merge their (max, sum, O) triples through LDS,
-// workgroups write one partial per (group, split), and then every workgroup merges one slice of the
-// output from all partials of its group as soon as they have arrived, in the same launch.
+// nsplit workgroups x 4 wavefronts.  A wave is on its own until its tiles are done: it issues the
+// few loads of the group's query rows first, then the 32 loads of a whole tile (16 KiB of K rows and
+// 16 KiB of V columns, streaming loads), and ropes, scales and rounds the queries in registers while
+// the tile is in flight; nothing goes through LDS and no wave waits for another one.  The up to 16
+// query heads of the group are the 16 columns of v_mfma_f32_16x16x32_f16 tiles: S^T = K q^T puts keys
+// on the rows, which is exactly the layout the second product O^T = V^T P^T wants for P^T, so
+// probabilities go from accumulator registers to operand registers without touching LDS.
+//
+// The four waves of a workgroup merge their (max, sum, O) through LDS.  Across workgroups the merge
+// happens in the same launch: every workgroup leaves its partial in memory as self-validating 64-byte
+// lines, one per (head, 16 output dims), and one wave of every workgroup then folds the lines of all
+// splits for one such slice of the output.
 //
 // The new token's K and V never take part in a cache load of this launch: one wave of each group
-// ropes them, stores them to the cache and feeds them to the same tile code through LDS.
+// ropes them, stores them to the cache and starts its softmax state from them, all in registers.
 #include "glm_attn_internal.h"
 
 namespace glm_attn {
+
+#ifdef GLM_ATTN_TIMELINE
+// Instrumented build (csrc/Makefile, target `timeline`): every wave leaves 100 MHz clock readings here.
+__device__ unsigned long long g_decode_timeline[kTimelineSlots * 16];
+#define TS(i)                                                                                                \
+    do {                                                                                                     \
+        const int slot_ = (blockIdx.y * gridDim.x + blockIdx.x) * 2 * kDecodeMaxWaves + (threadIdx.x >> 6);      \
+        if ((threadIdx.x & 63) == 0 && slot_ < kTimelineSlots) g_decode_timeline[slot_ * 16 + (i)] = wall_clock64(); \
+    } while (0)
+#else
+#define TS(i) \
+    do {      \
+    } while (0)
+#endif
 
 namespace {
 
 constexpr int D = kFastHeadSize;
 constexpr int TILE = kDecodeTileKeys;
-constexpr int OPAD = D + 4;  // row pitch of the per-wave O tile in LDS (floats)
-constexpr int kMaxSplits = kDecodeMaxSplits;
-constexpr int CHUNKS = kDecodePartFloats / 64;  // 16-byte records per head in a split partial
-constexpr int O_CHUNKS = CHUNKS - 1;            // ... of which the first 32 hold O, four dims each
-constexpr int ML_CHUNK = CHUNKS - 1;            // ... and the last one (max, sum)
-static_assert(O_CHUNKS * 4 == D, "record layout");
+constexpr int W = kDecodeMaxWaves;
+constexpr int QUADS = D / 16;  // 16-dim slices of a head: one 64-byte line each in a split partial
+static_assert(kDecodePartFloats == kMaxGroupHeads * QUADS * 16, "line layout");
 
-// Data that crosses workgroups inside one launch (split partials, hand-over words) moves with relaxed
-// device-scope accesses: they are performed at the device's coherence point, so neither side needs a
-// device-scope fence.  Such fences write back or invalidate a whole L2 on this multi-die part and
-// cost far more than the data they would publish.
-// 16-byte store at device scope.  The compiler does not count this store, so callers wait with
-// wait_stores_dev() before they tell other workgroups about the data.
 typedef unsigned int uintx4 __attribute__((ext_vector_type(4)));
 
-// A record of a split partial: the launch stamp and four floats cut to their upper three bytes (sign,
-// exponent and 15 mantissa bits, rounded to nearest: 2^-17 relative, far below what the fp16 products
-// feeding O carry).  NaNs are made quiet instead of rounded, so that they stay NaNs.
-__device__ inline unsigned int round24(float x) {
+// ---------------------------------------------------------------------------------------------------
+// Lines of a split partial.  A line is four 16-byte pieces; piece p holds the launch's stamp, four
+// values of O / sum cut to 22 bits (sign, exponent, 13 mantissa bits, rounded to nearest: 2^-14
+// relative on values that are averages of V) and byte p of the fp32 log-sum-exp max + ln(sum) of the
+// (split, head).  A 16-byte store is performed as one, so a piece that shows the stamp is complete:
+// the data is its own ready flag.
+__device__ inline unsigned int round22(float x) {
     const unsigned int u = __float_as_uint(x);
-    return x != x ? (u | 0x00400000u) : u + 0x80u;
+    return x != x ? ((u | 0x00400000u) >> 10) : ((u + 0x200u) >> 10);
 }
-__device__ inline uintx4 pack_record(unsigned int stamp, floatx4 v) {
-    const unsigned int a = round24(v[0]), b = round24(v[1]), c = round24(v[2]), d = round24(v[3]);
-    return uintx4{stamp, __builtin_amdgcn_perm(a, b, 0x07060503u), __builtin_amdgcn_perm(b, c, 0x06050302u),
-                  __builtin_amdgcn_perm(c, d, 0x05030201u)};
+__device__ inline uintx4 pack_piece(unsigned int stamp, floatx4 v, unsigned int lse_bits, int p) {
+    const unsigned int a = round22(v[0]), b = round22(v[1]), c = round22(v[2]), d = round22(v[3]);
+    const unsigned int lse_byte = (lse_bits >> (8 * p)) & 0xffu;
+    return uintx4{stamp, a | (b << 22), (b >> 10) | (c << 12), (c >> 20) | (d << 2) | (lse_byte << 24)};
 }
-__device__ inline floatx4 unpack_record(uintx4 r) {
-    return floatx4{__uint_as_float(r[1] & 0xffffff00u), __uint_as_float(__builtin_amdgcn_perm(r[1], r[2], 0x0403020cu)),
-                   __uint_as_float(__builtin_amdgcn_perm(r[2], r[3], 0x0504030cu)), __uint_as_float(r[3] << 8)};
+__device__ inline floatx4 unpack_piece(uintx4 r) {
+    const unsigned int a = r[1] & 0x3fffffu, b = (r[1] >> 22) | ((r[2] & 0xfffu) << 10);
+    const unsigned int c = (r[2] >> 12) | ((r[3] & 3u) << 20), d = (r[3] >> 2) & 0x3fffffu;
+    return floatx4{__uint_as_float(a << 10), __uint_as_float(b << 10), __uint_as_float(c << 10),
+                   __uint_as_float(d << 10)};
 }
 
+// Data that crosses workgroups inside one launch moves with relaxed device-scope accesses: they are
+// performed at the device's coherence point, so neither side needs a device-scope fence (such fences
+// write back or invalidate a whole L2 on this multi-die part and cost far more than the data).
+// (The s_nop covers the wait state that the hardware wants between a store of more than 8 bytes and a
+// write to the registers that hold its data: the compiler does not look into the assembly.)
 __device__ inline void st_dev4(float *p, uintx4 v) {
-    asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(p), "v"(v) : "memory");
+    asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" : : "v"(p), "v"(v) : "memory");
 }
-__device__ inline void wait_stores_dev() { asm volatile("s_waitcnt vmcnt(0)" : : : "memory"); }
+__device__ inline void wait_vm() { asm volatile("s_waitcnt vmcnt(0)" : : : "memory"); }
 
-// Up to four 16-byte loads at device scope, all issued before the one wait.  Pair u (pa[u], pb[u]) is
-// loaded by the lanes whose bit is set in mask[u]; the other lanes keep what va[u], vb[u] held.
-__device__ inline void ld_dev4x4(const float *const (&pa)[2], const float *const (&pb)[2], uintx4 (&va)[2],
-                                 uintx4 (&vb)[2], const unsigned long long (&mask)[2]) {
+// Eight 16-byte loads at device scope, all issued before the one wait.  Load i is done by the lanes
+// whose bit is set in mask[i]; the other lanes keep what r[i] held.  One block of assembly, so that
+// nothing can touch the destination registers between the loads and the wait.
+__device__ inline void ld_lines8(const float *const (&p)[8], uintx4 (&r)[8], const unsigned long long (&m)[8]) {
     unsigned long long saved;
     asm volatile("s_mov_b64 %[sv], exec\n\t"
                  "s_and_b64 exec, %[sv], %[m0]\n\t"
-                 "global_load_dwordx4 %[a0], %[pa0], off sc1\n\t"
-                 "global_load_dwordx4 %[b0], %[pb0], off sc1\n\t"
+                 "global_load_dwordx4 %[r0], %[p0], off sc1\n\t"
                  "s_and_b64 exec, %[sv], %[m1]\n\t"
-                 "global_load_dwordx4 %[a1], %[pa1], off sc1\n\t"
-                 "global_load_dwordx4 %[b1], %[pb1], off sc1\n\t"
+                 "global_load_dwordx4 %[r1], %[p1], off sc1\n\t"
+                 "s_and_b64 exec, %[sv], %[m2]\n\t"
+                 "global_load_dwordx4 %[r2], %[p2], off sc1\n\t"
+                 "s_and_b64 exec, %[sv], %[m3]\n\t"
+                 "global_load_dwordx4 %[r3], %[p3], off sc1\n\t"
+                 "s_and_b64 exec, %[sv], %[m4]\n\t"
+                 "global_load_dwordx4 %[r4], %[p4], off sc1\n\t"
+                 "s_and_b64 exec, %[sv], %[m5]\n\t"
+                 "global_load_dwordx4 %[r5], %[p5], off sc1\n\t"
+                 "s_and_b64 exec, %[sv], %[m6]\n\t"
+                 "global_load_dwordx4 %[r6], %[p6], off sc1\n\t"
+                 "s_and_b64 exec, %[sv], %[m7]\n\t"
+                 "global_load_dwordx4 %[r7], %[p7], off sc1\n\t"
                  "s_mov_b64 exec, %[sv]\n\t"
                  "s_waitcnt vmcnt(0)"
-                 : [sv] "=&s"(saved), [a0] "+v"(va[0]), [a1] "+v"(va[1]), [b0] "+v"(vb[0]), [b1] "+v"(vb[1])
-                 : [pa0] "v"(pa[0]), [pa1] "v"(pa[1]), [pb0] "v"(pb[0]), [pb1] "v"(pb[1]), [m0] "s"(mask[0]),
-                   [m1] "s"(mask[1])
+                 : [sv] "=&s"(saved), [r0] "+v"(r[0]), [r1] "+v"(r[1]), [r2] "+v"(r[2]), [r3] "+v"(r[3]),
+                   [r4] "+v"(r[4]), [r5] "+v"(r[5]), [r6] "+v"(r[6]), [r7] "+v"(r[7])
+                 : [p0] "v"(p[0]), [p1] "v"(p[1]), [p2] "v"(p[2]), [p3] "v"(p[3]), [p4] "v"(p[4]), [p5] "v"(p[5]),
+                   [p6] "v"(p[6]), [p7] "v"(p[7]), [m0] "s"(m[0]), [m1] "s"(m[1]), [m2] "s"(m[2]), [m3] "s"(m[3]),
+                   [m4] "s"(m[4]), [m5] "s"(m[5]), [m6] "s"(m[6]), [m7] "s"(m[7])
                  : "memory", "scc");
 }
-
-// A softmax partial of four output dims: running max, sum of exp and unnormalised O at that max.
-struct Partial {
-    float m;
-    float l;
-    floatx4 o;
-};
-
-__device__ inline Partial merge_partials(const Partial &x, const Partial &y) {
-    const float m = fmaxf(x.m, y.m);
-    const float fx = (x.m == -INFINITY) ? 0.f : __expf(x.m - m);
-    const float fy = (y.m == -INFINITY) ? 0.f : __expf(y.m - m);
-    Partial r;
-    r.m = m;
-    r.l = __builtin_fmaf(x.l, fx, y.l * fy);
-#pragma unroll
-    for (int e = 0; e < 4; e++) {
-        r.o[e] = __builtin_fmaf(x.o[e], fx, y.o[e] * fy);
-    }
-    return r;
-}
-
-// The value N lanes down within each row of 16 lanes; lanes without such a neighbour get `none`.
-template <int N>
-__device__ inline float row_shr_f(float v, float none) {
-    return __int_as_float(
-        __builtin_amdgcn_update_dpp(__float_as_int(none), __float_as_int(v), 0x110 + N, 0xf, 0xf, false));
-}
-template <int N>
-__device__ inline Partial row_shr(const Partial &x) {
-    Partial r;
-    r.m = row_shr_f<N>(x.m, -INFINITY);
-    r.l = row_shr_f<N>(x.l, 0.f);
-#pragma unroll
-    for (int e = 0; e < 4; e++) {
-        r.o[e] = row_shr_f<N>(x.o[e], 0.f);
-    }
-    return r;
-}
-__device__ inline Partial lane_xor(const Partial &x, int mask) {
-    Partial r;
-    r.m = __shfl_xor(x.m, mask);
-    r.l = __shfl_xor(x.l, mask);
-#pragma unroll
-    for (int e = 0; e < 4; e++) {
-        r.o[e] = __shfl_xor(x.o[e], mask);
-    }
-    return r;
-}
-
-struct WaveState {
-    float m;         // running max of this lane's head (column lane & 15)
-    float l;         // running sum of exp
-    floatx4 o[8];    // O^T[dim = jb*16 + (lane>>4)*4 + r][head = lane & 15]
-};
 
 __device__ inline floatx4 mfma16(half8 a, half8 b, floatx4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
 }
 
-// Row rho (0..15) of sub-block T (0..3) of a 64-key tile holds this key of the tile.  The order is
-// chosen so that accumulator row 4c + r of sub-block T is element (T & 1) * 4 + r of k-slice c of
-// the 32-key step T >> 1 of the second product.
+// Row rho (0..15) of sub-block T (0..3) of a 64-key tile holds this key of the tile: accumulator row
+// 4c + r of sub-block T is key (T >> 1) * 32 + c * 8 + (T & 1) * 4 + r, so that a lane's eight values
+// of sub-blocks 2u and 2u + 1 are eight consecutive keys, one 16-byte piece of the P operand.
 __device__ inline int tile_key(int T, int rho) { return (T >> 1) * 32 + (rho >> 2) * 8 + (T & 1) * 4 + (rho & 3); }
 
-__device__ inline void load_tile(const __half *Kg, const __half *Vg, int L, int key0, int lane, half8 (&kf)[4][4],
-                                 half8 (&vf)[8][2]) {
+__device__ inline half8 ld_stream(const __half *p) { return *reinterpret_cast<const half8 *>(p); }
+
+// K rows of one 64-key tile as MFMA A operands: lane (j, c) holds dims t*32 + c*8 .. of key tile_key(T, j).
+__device__ inline void load_k_tile(const __half *Kg, int L, int key0, int lane, half8 (&kf)[4][4]) {
     const int j = lane & 15, c = lane >> 4;
 #pragma unroll
     for (int T = 0; T < 4; T++) {
@@ -152,710 +130,746 @@ __device__ inline void load_tile(const __half *Kg, const __half *Vg, int L, int 
         const __half *row = Kg + (int64_t)key * D + c * 8;
 #pragma unroll
         for (int t = 0; t < 4; t++) {
-            kf[T][t] = *reinterpret_cast<const half8 *>(row + t * 32);
-        }
-    }
-#pragma unroll
-    for (int u = 0; u < 2; u++) {
-        int s0 = key0 + u * 32 + c * 8;
-        s0 = s0 <= L - 8 ? s0 : L - 8;
-#pragma unroll
-        for (int jb = 0; jb < 8; jb++) {
-            vf[jb][u] = *reinterpret_cast<const half8 *>(Vg + (int64_t)(jb * 16 + j) * L + s0);
+            kf[T][t] = ld_stream(row + t * 32);
         }
     }
 }
 
-// One 64-key tile: S^T = K q^T, online softmax against the wave's running state, O^T += V^T P^T.
-// Keys of the tile with index >= limit do not exist (tail of the sequence) and are masked.
-__device__ inline void process_tile(const half8 (&kf)[4][4], half8 (&vf)[8][2], const half8 (&qf)[4], int limit,
-                                    int lane, WaveState &st) {
-    const int c = lane >> 4;
-    floatx4 s[4];
+// V columns of up to 256 keys (nk tiles from key0) for the 32 output dims of wave w, as MFMA A operands:
+// lane (j, c) holds keys ks*32 + c*8 .. of dim w*32 + jb*16 + j.  Steps beyond the nk tiles read step 0
+// again (the same lines, no extra memory traffic) and are not used.
+template <int KS0, int KS1>
+__device__ inline void load_v_dims(const __half *Vg, int L, int key0, int nk, int w, int lane, half8 (&vf)[2][8]) {
+    const int j = lane & 15, c = lane >> 4;
 #pragma unroll
-    for (int T = 0; T < 4; T++) {
+    for (int jb = 0; jb < 2; jb++) {
+        const __half *row = Vg + (int64_t)(w * 32 + jb * 16 + j) * L;
+#pragma unroll
+        for (int ks = KS0; ks < KS1; ks++) {
+            int s0 = key0 + (ks < 2 * nk ? ks : 0) * 32 + c * 8;
+            s0 = s0 <= L - 8 ? s0 : L - 8;
+            vf[jb][ks] = ld_stream(row + s0);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------
+// A head's row in the registers of one lane, in the MFMA operand layout: lane (j, c) holds dims
+// t*32 + c*8 + e, t = 0..3, e = 0..7.  For every rope type the partner of each of these 32 dims is
+// one of them too, so a lane ropes its share on its own.  The cos/sin pairs it needs are contiguous in
+// a table row and are fetched with 16-byte loads (two pairs each).
+struct RowRegs {
+    floatx4 x[4][2];
+    floatx4 cs[8];
+};
+
+template <int TYPE>
+__device__ inline void issue_row_loads(const float *head, int c, const int (&pos)[2], const RopeSpec &rope,
+                                       RowRegs &r) {
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+        r.x[t][0] = *reinterpret_cast<const floatx4 *>(head + t * 32 + c * 8);
+        r.x[t][1] = *reinterpret_cast<const floatx4 *>(head + t * 32 + c * 8 + 4);
+    }
+    if (TYPE == GLM_ATTN_ROPE_GPTJ || TYPE == GLM_ATTN_ROPE_CHATGLM2) {
+        // pair of dim d is d >> 1: four pairs per t, from t*16 + c*4
+        constexpr int NT = (TYPE == GLM_ATTN_ROPE_GPTJ) ? 4 : 2;
+        const float2 *row = rope.table + (int64_t)pos[0] * rope.pairs;
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            r.cs[t * 2 + 0] = *reinterpret_cast<const floatx4 *>(row + t * 16 + c * 4);
+            r.cs[t * 2 + 1] = *reinterpret_cast<const floatx4 *>(row + t * 16 + c * 4 + 2);
+        }
+    } else if (TYPE == GLM_ATTN_ROPE_NEOX) {
+        // pair of dim d is d % 64: eight pairs from (t & 1)*32 + c*8, shared by t and t + 2
+        const float2 *row = rope.table + (int64_t)pos[0] * rope.pairs;
+#pragma unroll
+        for (int tt = 0; tt < 2; tt++) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                r.cs[tt * 4 + i] = *reinterpret_cast<const floatx4 *>(row + tt * 32 + c * 8 + i * 2);
+            }
+        }
+    } else if (TYPE == GLM_ATTN_ROPE_CHATGLM) {
+        // NEOX inside each half of the head: pair c*8 + e for both t of a half, positions per half
+#pragma unroll
+        for (int hf = 0; hf < 2; hf++) {
+            const float2 *row = rope.table + (int64_t)pos[hf] * rope.pairs;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                r.cs[hf * 4 + i] = *reinterpret_cast<const floatx4 *>(row + c * 8 + i * 2);
+            }
+        }
+    }
+}
+
+// rope (chatglm.cpp:523-618), then `* scale` in fp32 and the fp16 rounding of ggml's mat-mul operand
+template <int TYPE>
+__device__ inline void finish_row(const RowRegs &r, float scale, bool zero, half8 (&out)[4]) {
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            const float self = r.x[t][e >> 2][e & 3];
+            float x = self;
+            if (TYPE == GLM_ATTN_ROPE_GPTJ || (TYPE == GLM_ATTN_ROPE_CHATGLM2 && t < 2)) {
+                const float partner = r.x[t][e >> 2][(e & 3) ^ 1];
+                const floatx4 cs = r.cs[t * 2 + (e >> 2)];
+                const int k = (e >> 1) & 1;
+                x = rope_rotate(self, partner, cs[2 * k], cs[2 * k + 1], !(e & 1));
+            } else if (TYPE == GLM_ATTN_ROPE_NEOX) {
+                const float partner = r.x[t ^ 2][e >> 2][e & 3];
+                const floatx4 cs = r.cs[(t & 1) * 4 + (e >> 1)];
+                x = rope_rotate(self, partner, cs[2 * (e & 1)], cs[2 * (e & 1) + 1], t < 2);
+            } else if (TYPE == GLM_ATTN_ROPE_CHATGLM) {
+                const float partner = r.x[t ^ 1][e >> 2][e & 3];
+                const floatx4 cs = r.cs[(t >> 1) * 4 + (e >> 1)];
+                x = rope_rotate(self, partner, cs[2 * (e & 1)], cs[2 * (e & 1) + 1], !(t & 1));
+            }
+            out[t][e] = zero ? (_Float16)0.f : (_Float16)__fmul_rn(x, scale);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Merge across workgroups: fold the lines of all splits for quads [q_begin, q_end) of KV group g.
+// Quads are dealt out to the calling waves (wave `wi` of `nw`), `qw` of them at a time per wave: lane
+// (qslot, s, piece) takes piece `piece` of the lines of splits s, s + SL, ... of its quad.
+struct MergeGeom {
+    int nsplit, G, sl_log;  // SL = 1 << sl_log lanes per (quad, piece)
+    unsigned int stamp32;
+    const float *part_g;    // lines of the group: [nsplit][16 heads][QUADS][16 floats]
+    float *out_g;           // [G][D]
+};
+
+// All-lanes reductions over the lanes that differ in bits [2, 2 + sl_log) of the lane index.  With 16
+// such lanes (the long-context shape) they need no LDS: two rotations inside the rows of 16 lanes fused
+// into the operation (DPP), then the two row swaps of gfx950.
+__device__ inline float rot_row(float x, int n) {
+    return n == 4 ? __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x124, 0xf, 0xf, false))
+                  : __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x128, 0xf, 0xf, false));
+}
+template <typename F>
+__device__ inline float reduce_splits(float x, int sl_log, F op) {
+    if (sl_log == 4) {
+        x = op(x, rot_row(x, 4));
+        x = op(x, rot_row(x, 8));
+        auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+        x = op(__uint_as_float(a[0]), __uint_as_float(a[1]));
+        auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+        return op(__uint_as_float(b[0]), __uint_as_float(b[1]));
+    }
+    if (sl_log > 0) x = op(x, __shfl_xor(x, 4));
+    if (sl_log > 1) x = op(x, __shfl_xor(x, 8));
+    if (sl_log > 2) x = op(x, __shfl_xor(x, 16));
+    return x;
+}
+
+// Returns 0 when every quad was written, 1 when the wait ran out (nothing is written for that pass).
+__device__ inline int merge_quads(const MergeGeom &mg, int q_begin, int q_end, int wi, int nw, int lane,
+                                  unsigned long long t0, unsigned long long limit) {
+    const int SL = 1 << mg.sl_log, qw = 16 >> mg.sl_log;
+    const int piece = lane & 3, s = (lane >> 2) & (SL - 1), qslot = lane >> (2 + mg.sl_log);
+    for (int q0 = q_begin + wi * qw; q0 < q_end; q0 += nw * qw) {
+        const int q = q0 + qslot;
+        const bool valid = q < q_end;
+        const int qc = valid ? q : q_end - 1;
+        const int hd = qc / QUADS, quad = qc - hd * QUADS;
+        const float *base = mg.part_g + ((hd * QUADS + quad) * 4 + piece) * 4;
+        float run_m = -INFINITY, acc_w = 0.f;
+        floatx4 acc_o = {0.f, 0.f, 0.f, 0.f};
+        for (int b0 = 0; b0 < mg.nsplit; b0 += 8 * SL) {
+            uintx4 r[8];
+            const float *p[8];
+            bool need[8];
+            unsigned long long stale[8];
+#pragma unroll
+            for (int it = 0; it < 8; it++) {
+                const int sp = b0 + it * SL + s;
+                r[it] = uintx4{0u, 0u, 0u, 0u};
+                need[it] = valid && sp < mg.nsplit;
+                p[it] = base + (int64_t)(sp < mg.nsplit ? sp : 0) * kDecodePartFloats;
+                stale[it] = __ballot(need[it]);
+            }
+            while (true) {
+                ld_lines8(p, r, stale);  // only what has not arrived yet is loaded again
+                unsigned long long any = 0ull;
+#pragma unroll
+                for (int it = 0; it < 8; it++) {
+                    stale[it] = __ballot(need[it] && r[it][0] != mg.stamp32);
+                    any |= stale[it];
+                }
+                if (any == 0ull) {
+                    break;
+                }
+                if (wall_clock64() - t0 > limit) {
+                    return 1;
+                }
+                __builtin_amdgcn_s_sleep(2);
+            }
+            // log-sum-exp of each line from the bytes in its four pieces, then the batch's max
+            float lse[8];
+            float bm = -INFINITY;
+#pragma unroll
+            for (int it = 0; it < 8; it++) {
+                int bits = (int)(r[it][3] >> 24) << (8 * piece);
+                bits |= __builtin_amdgcn_update_dpp(0, bits, 0xB1, 0xf, 0xf, true);  // quad_perm [1,0,3,2]
+                bits |= __builtin_amdgcn_update_dpp(0, bits, 0x4E, 0xf, 0xf, true);  // quad_perm [2,3,0,1]
+                lse[it] = need[it] ? __int_as_float(bits) : -INFINITY;
+                bm = fmaxf(bm, lse[it]);
+            }
+            bm = reduce_splits(bm, mg.sl_log, [](float a, float b) { return fmaxf(a, b); });
+            const float m_new = fmaxf(run_m, bm);
+            if (m_new != -INFINITY) {
+                const float sc = (run_m == -INFINITY) ? 0.f : __expf(run_m - m_new);
+                acc_w *= sc;
+                acc_o *= sc;
+#pragma unroll
+                for (int it = 0; it < 8; it++) {
+                    const float wgt = (lse[it] == -INFINITY) ? 0.f : __expf(lse[it] - m_new);
+                    const floatx4 v = unpack_piece(r[it]);
+                    acc_w += wgt;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        acc_o[e] = __builtin_fmaf(wgt, v[e], acc_o[e]);
+                    }
+                }
+                run_m = m_new;
+            }
+        }
+        auto add = [](float a, float b) { return a + b; };
+        acc_w = reduce_splits(acc_w, mg.sl_log, add);
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            acc_o[e] = reduce_splits(acc_o[e], mg.sl_log, add);
+        }
+        if (valid && s == 0) {
+            // (1 / sum to one ulp, then a product: the values were cut to 22 bits on their way here)
+            *reinterpret_cast<floatx4 *>(mg.out_g + hd * D + quad * 16 + piece * 4) =
+                acc_o * __builtin_amdgcn_rcpf(acc_w);
+        }
+    }
+    return 0;
+}
+
+#ifndef EXP_DELAY_DIV
+#define EXP_DELAY_DIV 8
+#endif
+#ifndef EXP_DELAY_ADD
+#define EXP_DELAY_ADD 30
+#endif
+constexpr int PPITCH = W * TILE + 8;  // row pitch of the P tile in LDS (halfs): conflict-free 16-byte accesses
+constexpr int kBlock = 2 * W * 64;    // W score waves, then W output waves
+
+struct DecodeShared {
+    __attribute__((aligned(16))) __half p[16][PPITCH];  // P^T of the round: [head][key]
+    float m[2][W][16];  // maxes of a round per score wave (rounds alternate between the two copies)
+    float mrun[2][16];  // running max after a round
+    float l[W][16];     // sums per score wave, at the final running max
+    float pnew[16];     // probability of the new token
+    int m_ready;        // score waves that have left their maxes, over all rounds
+    int p_ready;        // score waves that have left their part of P, over all rounds
+    int p_done;         // output waves that are through with P, over all rounds
+    int stored;         // output waves whose line stores have been performed
+};
+
+// A wave waits for waves of its own workgroup (all resident by construction) through a counter in LDS.
+// The wait is bounded all the same, so that a mistake in the hand-over could not hang the device: when
+// it runs out the launch goes on with what it has and reports it.
+__device__ inline void lds_wait_ge(int *ctr, int target, uint32_t *flags) {
+    for (int i = 0; i < (1 << 20); i++) {
+        if (__hip_atomic_load(ctr, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) >= target) {
+            return;
+        }
+        __builtin_amdgcn_s_sleep(1);
+    }
+    atomicOr(flags, kFlagMergeIncomplete);
+}
+__device__ inline void lds_signal(int *ctr, int lane) {
+    // the wave's LDS writes first, then the count
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    if (lane == 0) {
+        __hip_atomic_fetch_add(ctr, 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
+}
+
+__device__ inline float max_over_c(float x) {  // over the four lanes (j, c) of a head
+    auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    x = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+    auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+__device__ inline float sum_over_c(float x) {
+    auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    x = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+    auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+
+struct Geom {
+    int lane, w, j, c, g, split;
+    int tb, te, rounds;
+    bool owner_wg;
+    unsigned long long t_start;
+};
+
+// ---- score waves: S^T = K q^T of one tile per round, the softmax across the workgroup's tiles, P to LDS
+template <int TYPE>
+__device__ inline void score_wave(const DecodeArgs &a, DecodeShared &sh, const Geom &ge) {
+    const int lane = ge.lane, w = ge.w, j = ge.j, c = ge.c, g = ge.g;
+    const int L = a.s.L, G = a.s.G;
+    const __half *Kg = a.k_cache + (int64_t)g * L * D;
+    const bool owner = ge.owner_wg && w == 0;
+
+    int nk = ge.te - ge.tb < W ? ge.te - ge.tb : W;
+    half8 kf[4][4];
+    load_k_tile(Kg, L, (ge.tb + (w < nk ? w : 0)) * TILE, lane, kf);
+    int pos[2] = {a.pos0, a.pos1};
+    if (TYPE != GLM_ATTN_ROPE_DISABLED) {
+        if (!a.pos_from_args) {
+            pos[0] = a.position_ids[0];
+            pos[1] = (TYPE == GLM_ATTN_ROPE_CHATGLM) ? a.position_ids[1] : 0;
+        }
+        pos[0] = clamp_position(pos[0], a.rope.table_positions, a.flags);
+        pos[1] = clamp_position(pos[1], a.rope.table_positions, a.flags);
+    }
+    RowRegs qreg;
+    {
+        const int hd = j < G ? j : G - 1;  // lanes beyond the group read a valid row and are zeroed below
+        issue_row_loads<TYPE>(a.qkv + a.lay.q_off + (int64_t)(g * G + hd) * a.lay.head_stride, c, pos, a.rope, qreg);
+    }
+    RowRegs kreg;
+    if (owner) {
+        issue_row_loads<TYPE>(a.qkv + a.lay.k_off + (int64_t)g * a.lay.head_stride, c, pos, a.rope, kreg);
+    }
+    TS(0);
+    half8 qf[4];
+    finish_row<TYPE>(qreg, a.scale, j >= G, qf);
+    float s_new = -INFINITY;  // score of the new token, in the wave that attends to it
+    if (owner) {
+        // chatglm.cpp:668-671: k (roped) of the new token goes to the cache as fp16
+        half8 kn[4];
+        finish_row<TYPE>(kreg, 1.0f, false, kn);
+        const half8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
         floatx4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int t = 0; t < 4; t++) {
-            acc = mfma16(kf[T][t], qf[t], acc);
+            if (j == 0) {
+                *reinterpret_cast<half8 *>(a.k_cache + ((int64_t)g * L + a.p0) * D + t * 32 + c * 8) = kn[t];
+            }
+            acc = mfma16(j == 0 ? kn[t] : zero, qf[t], acc);  // row 0 of the product: the new key
         }
-        s[T] = acc;
+        s_new = __shfl(acc[0], j);
     }
-    float mx = -INFINITY;
-    if (limit < TILE) {
+    TS(1);
+
+    float m_run = -INFINITY, l_run = 0.f;
+    for (int r = 0; r < ge.rounds; r++) {
+        const int rt0 = ge.tb + r * W;  // first tile of the round
+        if (r > 0) {
+            nk = ge.te - rt0 < W ? ge.te - rt0 : W;
+            load_k_tile(Kg, L, (rt0 + (w < nk ? w : 0)) * TILE, lane, kf);
+        }
+        const bool has = w < nk;
+        floatx4 s[4];
 #pragma unroll
         for (int T = 0; T < 4; T++) {
-#pragma unroll
-            for (int r = 0; r < 4; r++) {
-                const int k = (T >> 1) * 32 + c * 8 + (T & 1) * 4 + r;
-                if (k >= limit) {
-                    s[T][r] = -INFINITY;
-                }
-            }
-        }
-        // V columns of missing keys may hold anything (never written, or stale): zero them
-#pragma unroll
-        for (int u = 0; u < 2; u++) {
-#pragma unroll
-            for (int e = 0; e < 8; e++) {
-                if (u * 32 + c * 8 + e >= limit) {
-#pragma unroll
-                    for (int jb = 0; jb < 8; jb++) {
-                        vf[jb][u][e] = (_Float16)0.f;
-                    }
-                }
-            }
-        }
-    }
-#pragma unroll
-    for (int T = 0; T < 4; T++) {
-#pragma unroll
-        for (int r = 0; r < 4; r++) {
-            mx = fmaxf(mx, s[T][r]);
-        }
-    }
-    mx = fmaxf(mx, __shfl_xor(mx, 16));
-    mx = fmaxf(mx, __shfl_xor(mx, 32));
-    const float m_new = fmaxf(st.m, mx);
-    const float m_ref = (m_new == -INFINITY) ? 0.f : m_new;  // no visible key yet: every p below is 0
-    const float alpha = (st.m == -INFINITY) ? 0.f : __expf(st.m - m_ref);
-    float psum = 0.f;
-    half8 pf[2];
-#pragma unroll
-    for (int T = 0; T < 4; T++) {
-#pragma unroll
-        for (int r = 0; r < 4; r++) {
-            const float p = __expf(s[T][r] - m_ref);  // exp(-inf) = 0 for masked keys
-            psum += p;
-            pf[T >> 1][(T & 1) * 4 + r] = (_Float16)p;
-        }
-    }
-    psum += __shfl_xor(psum, 16);
-    psum += __shfl_xor(psum, 32);
-    st.l = st.l * alpha + psum;
-    st.m = m_new;
-#pragma unroll
-    for (int jb = 0; jb < 8; jb++) {
-        floatx4 acc = st.o[jb] * alpha;
-        acc = mfma16(vf[jb][0], pf[0], acc);
-        acc = mfma16(vf[jb][1], pf[1], acc);
-        st.o[jb] = acc;
-    }
-}
-
-constexpr int QPAD = D + 8;  // row pitch of the fp16 query tile in LDS (halfs): conflict-free b128 reads
-
-// The prep wave's work, specialised per rope type so that the pairing arithmetic folds to constants
-// and every load of a batch is issued before the first one is waited for.
-//
-// 16 heads x 128 dims are handled in groups of 4 consecutive dims: 512 groups, 8 per lane.
-template <int TYPE>
-__device__ inline void prep_queries(const DecodeArgs &a, int g, int lane, const int (&pos)[2], __half (*q_s)[QPAD]) {
-    constexpr bool kRope = (TYPE != GLM_ATTN_ROPE_DISABLED);
-    constexpr bool kAdjacent = (TYPE == GLM_ATTN_ROPE_GPTJ || TYPE == GLM_ATTN_ROPE_CHATGLM2);
-    const int G = a.s.G;
-    {
-        constexpr int NB = 8;
-        floatx4 x4[NB], p4[NB];
-        float2 cs[NB][4];
-#pragma unroll
-        for (int i = 0; i < NB; i++) {
-            const int grp = i * 64 + lane;
-            const int hd = grp >> 5, d0 = (grp & 31) * 4;
-            const int hd_ld = hd < G ? hd : G - 1;  // heads beyond the group read a valid row and are zeroed below
-            const float *qhead = a.qkv + a.lay.q_off + (int64_t)(g * G + hd_ld) * a.lay.head_stride;
-            x4[i] = *reinterpret_cast<const floatx4 *>(qhead + d0);
-            if (kRope && !kAdjacent) {
-                p4[i] = *reinterpret_cast<const floatx4 *>(qhead + rope_elem(TYPE, D, d0).partner);
-            }
-            if (kRope) {
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    const RopeElem r = rope_elem(TYPE, D, d0 + e);
-                    const int64_t idx = r.rot ? (int64_t)pos[r.sel] * a.rope.pairs + r.pair : 0;
-                    cs[i][e] = a.rope.table[idx];
-                }
-            }
-        }
-#pragma unroll
-        for (int i = 0; i < NB; i++) {
-            const int grp = i * 64 + lane;
-            const int hd = grp >> 5, d0 = (grp & 31) * 4;
-            half4 q4;
-#pragma unroll
-            for (int e = 0; e < 4; e++) {
-                float x = x4[i][e];
-                if (kRope) {
-                    const RopeElem r = rope_elem(TYPE, D, d0 + e);
-                    const float partner = kAdjacent ? x4[i][e ^ 1] : p4[i][e];
-                    const float xr = rope_rotate(x, partner, cs[i][e].x, cs[i][e].y, r.first);
-                    x = r.rot ? xr : x;
-                }
-                // chatglm.cpp:686 scales q in fp32 after rope; the fp16 mat-mul rounds it to fp16
-                q4[e] = (hd < G) ? (_Float16)__fmul_rn(x, a.scale) : (_Float16)0.f;
-            }
-            *reinterpret_cast<half4 *>(&q_s[hd][d0]) = q4;
-        }
-    }
-}
-
-// The new token of KV group g: rope k, round k and v to fp16, store both to the cache
-// (chatglm.cpp:668-675) and leave them in LDS for the tile code.  Lane l handles dims l and l + 64.
-template <int TYPE>
-__device__ inline void prep_new_token(const DecodeArgs &a, int g, int lane, const int (&pos)[2], __half *new_k,
-                                      __half *new_v) {
-    constexpr bool kRope = (TYPE != GLM_ATTN_ROPE_DISABLED);
-    const int L = a.s.L;
-    const float *khead = a.qkv + a.lay.k_off + (int64_t)g * a.lay.head_stride;
-    const float *vhead = a.qkv + a.lay.v_off + (int64_t)g * a.lay.head_stride;
-    float x[2], xp[2], v[2];
-    float2 cs[2];
-#pragma unroll
-    for (int i = 0; i < 2; i++) {
-        const int e = lane + 64 * i;
-        const RopeElem r = rope_elem(TYPE, D, e);
-        x[i] = khead[e];
-        v[i] = vhead[e];
-        if (kRope) {
-            xp[i] = khead[r.partner];
-            cs[i] = a.rope.table[r.rot ? (int64_t)pos[r.sel] * a.rope.pairs + r.pair : 0];
-        }
-    }
-#pragma unroll
-    for (int i = 0; i < 2; i++) {
-        const int e = lane + 64 * i;
-        float k = x[i];
-        if (kRope) {
-            const RopeElem r = rope_elem(TYPE, D, e);
-            const float kr = rope_rotate(x[i], xp[i], cs[i].x, cs[i].y, r.first);
-            k = r.rot ? kr : k;
-        }
-        const __half k16 = __float2half_rn(k);
-        const __half v16 = __float2half_rn(v[i]);
-        new_k[e] = k16;
-        new_v[e] = v16;
-        a.k_cache[((int64_t)g * L + a.p0) * D + e] = k16;
-        a.v_cache[((int64_t)g * D + e) * L + a.p0] = v16;
-    }
-}
-
-template <int TYPE>
-__device__ inline void prep_wave(const DecodeArgs &a, int g, int lane, bool owner, const int (&pos)[2],
-                                 __half (*q_s)[QPAD], __half *new_k, __half *new_v) {
-    prep_queries<TYPE>(a, g, lane, pos, q_s);
-    if (owner) {
-        prep_new_token<TYPE>(a, g, lane, pos, new_k, new_v);
-    }
-}
-
-// Block = 1 prep wave + `waves` tile waves.  Tile waves issue their first tile's loads as their very
-// first instructions and only then wait for the prep wave, which meanwhile ropes, scales and rounds
-// the group's queries into LDS (and, in the owner workgroup, appends and attends to the new token).
-// Loads of one wave return in order, so anything a tile wave loaded after its tile would be usable
-// only after the whole tile had arrived; the prep wave keeps those small dependent loads out of the
-// tile waves' queues.
-__global__ __launch_bounds__((kDecodeMaxWaves + 1) * 64) void decode_kernel(DecodeArgs a) {
-    __shared__ __attribute__((aligned(16))) __half q_s[16][QPAD];
-    __shared__ __attribute__((aligned(16))) __half new_k[D];
-    __shared__ __attribute__((aligned(16))) __half new_v[D];
-    __shared__ float sm_m[kDecodeMaxWaves + 1][16];
-    __shared__ float sm_l[kDecodeMaxWaves + 1][16];
-    __shared__ float sm_mwg[16];
-    __shared__ __attribute__((aligned(16))) float sm_o[kDecodeMaxWaves + 1][16][OPAD];
-    __shared__ unsigned long long sh_gen;  // launches of this group completed before this one
-
-    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-    const int waves = a.waves;  // tile waves 1..waves have keys to read; wave 0 is the prep wave (it starts first)
-    const bool prep = (w == 0);
-    const int j = lane & 15, c = lane >> 4;
-    const int g = blockIdx.y, split = blockIdx.x;
-    const int L = a.s.L;
-    const __half *Kg = a.k_cache + (int64_t)g * L * D;
-    const __half *Vg = a.v_cache + (int64_t)g * D * L;
-
-    const int n_tiles = (a.p0 + TILE - 1) / TILE;  // tiles of keys already in the cache
-    const int nw = a.nsplit * waves;
-    const int wg = split * waves + (prep ? 0 : w - 1);
-    const bool reads = !prep && w <= waves;
-    const int tile_begin = reads ? (int)((int64_t)wg * n_tiles / nw) : 0;
-    const int tile_end = reads ? (int)((int64_t)(wg + 1) * n_tiles / nw) : 0;
-    const bool owner = prep && (split == a.nsplit - 1);  // appends the new token and attends to it
-
-    // the launch count stamps this launch's partials; read before any workgroup can have finished
-    unsigned long long my_gen = 0;
-    if (threadIdx.x == 0 && a.nsplit > 1) {
-        my_gen = __hip_atomic_load(a.sync_gen + g, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    half8 kf[4][4];
-    half8 vf[8][2];
-    if (tile_begin < tile_end) {
-        load_tile(Kg, Vg, L, tile_begin * TILE, lane, kf, vf);
-    }
-
-    if (prep) {
-        int pos[2] = {a.pos0, a.pos1};
-        if (a.rope.pairs > 0) {
-            if (!a.pos_from_args) {
-                pos[0] = a.position_ids[0];
-                pos[1] = (a.rope.type == GLM_ATTN_ROPE_CHATGLM) ? a.position_ids[1] : 0;
-            }
-            pos[0] = clamp_position(pos[0], a.rope.table_positions, a.flags);
-            pos[1] = clamp_position(pos[1], a.rope.table_positions, a.flags);
-        }
-        switch (a.rope.type) {
-        case GLM_ATTN_ROPE_GPTJ:
-            prep_wave<GLM_ATTN_ROPE_GPTJ>(a, g, lane, owner, pos, q_s, new_k, new_v);
-            break;
-        case GLM_ATTN_ROPE_NEOX:
-            prep_wave<GLM_ATTN_ROPE_NEOX>(a, g, lane, owner, pos, q_s, new_k, new_v);
-            break;
-        case GLM_ATTN_ROPE_CHATGLM:
-            prep_wave<GLM_ATTN_ROPE_CHATGLM>(a, g, lane, owner, pos, q_s, new_k, new_v);
-            break;
-        case GLM_ATTN_ROPE_CHATGLM2:
-            prep_wave<GLM_ATTN_ROPE_CHATGLM2>(a, g, lane, owner, pos, q_s, new_k, new_v);
-            break;
-        default:
-            prep_wave<GLM_ATTN_ROPE_DISABLED>(a, g, lane, owner, pos, q_s, new_k, new_v);
-            break;
-        }
-    }
-    if (threadIdx.x == 0) {
-        sh_gen = my_gen;
-    }
-    // Make the LDS writes of the prep wave visible without draining the tile loads in flight.
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
-    __builtin_amdgcn_s_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
-    half8 qf[4];
-#pragma unroll
-    for (int t = 0; t < 4; t++) {
-        qf[t] = *reinterpret_cast<const half8 *>(&q_s[j][t * 32 + c * 8]);
-    }
-
-    WaveState st;
-    st.m = -INFINITY;
-    st.l = 0.f;
-#pragma unroll
-    for (int jb = 0; jb < 8; jb++) {
-        st.o[jb] = floatx4{0.f, 0.f, 0.f, 0.f};
-    }
-
-    if (owner) {
-        // the new token as a tile whose only key is row 0 of sub-block 0, fed from LDS
-        const half8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
-#pragma unroll
-        for (int T = 0; T < 4; T++) {
+            floatx4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int t = 0; t < 4; t++) {
-                kf[T][t] = zero;
+                acc = mfma16(kf[T][t], qf[t], acc);
             }
+            s[T] = acc;
         }
+        const int limit = has ? a.p0 - (rt0 + w) * TILE : 0;  // keys of the tile that exist
+        if (limit < TILE) {
 #pragma unroll
-        for (int t = 0; t < 4; t++) {
-            const half8 kv = *reinterpret_cast<const half8 *>(&new_k[t * 32 + c * 8]);
-            kf[0][t] = (j == 0) ? kv : zero;
-        }
-#pragma unroll
-        for (int jb = 0; jb < 8; jb++) {
-            vf[jb][0] = zero;
-            vf[jb][1] = zero;
-            const _Float16 v = *reinterpret_cast<const _Float16 *>(&new_v[jb * 16 + j]);
-            vf[jb][0][0] = (c == 0) ? v : (_Float16)0.f;
-        }
-        process_tile(kf, vf, qf, 1, lane, st);
-    }
-
-    // ---- the cached keys of this wave
-    for (int tile = tile_begin; tile < tile_end; tile++) {
-        const int key0 = tile * TILE;
-        const int limit = a.p0 - key0 < TILE ? a.p0 - key0 : TILE;
-        process_tile(kf, vf, qf, limit, lane, st);
-        if (tile + 1 < tile_end) {
-            load_tile(Kg, Vg, L, key0 + TILE, lane, kf, vf);
-        }
-    }
-    // ---- merge the waves of this workgroup (tile waves and the prep wave): the maxes first, then
-    // every wave brings its sum and O to the workgroup's max before it leaves them in LDS.  The
-    // barriers wait for LDS only: the new token's cache stores may still be on their way.
-    constexpr int P = kDecodeMaxWaves + 1;  // waves of the block
-    if (c == 0) {
-        sm_m[w][j] = st.m;
-    }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
-    __builtin_amdgcn_s_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
-    {
-        float mw[P];
-#pragma unroll
-        for (int ww = 0; ww < P; ww++) {
-            mw[ww] = sm_m[ww][j];
-        }
-        float m_wg = mw[0];
-#pragma unroll
-        for (int ww = 1; ww < P; ww++) {
-            m_wg = fmaxf(m_wg, mw[ww]);
-        }
-        const float f = (st.m == -INFINITY) ? 0.f : __expf(st.m - m_wg);
-        if (c == 0) {
-            sm_l[w][j] = st.l * f;
-            if (w == 0) {
-                sm_mwg[j] = m_wg;
-            }
-        }
-#pragma unroll
-        for (int jb = 0; jb < 8; jb++) {
-            *reinterpret_cast<floatx4 *>(&sm_o[w][j][jb * 16 + c * 4]) = st.o[jb] * f;
-        }
-    }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
-    __builtin_amdgcn_s_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
-    // O of head hd, dims d4 .. d4 + 3, and the sum of head hd, over the waves
-    auto merged_o = [&](int hd, int d4) -> floatx4 {
-        floatx4 ow[P];
-#pragma unroll
-        for (int ww = 0; ww < P; ww++) {
-            ow[ww] = *reinterpret_cast<const floatx4 *>(&sm_o[ww][hd][d4]);
-        }
-        floatx4 acc = ow[0];
-#pragma unroll
-        for (int ww = 1; ww < P; ww++) {
-            acc += ow[ww];
-        }
-        return acc;
-    };
-    auto merged_l = [&](int hd) -> float {
-        float lw[P];
-#pragma unroll
-        for (int ww = 0; ww < P; ww++) {
-            lw[ww] = sm_l[ww][hd];
-        }
-        float l = lw[0];
-#pragma unroll
-        for (int ww = 1; ww < P; ww++) {
-            l += lw[ww];
-        }
-        return l;
-    };
-    const int tid = threadIdx.x;
-    if (a.nsplit == 1) {
-        // a single workgroup saw every key of the group: normalise and finish
-        for (int idx4 = tid; idx4 < a.s.G * (D / 4); idx4 += P * 64) {
-            const int hd = idx4 >> 5, d4 = (idx4 & 31) * 4;
-            const floatx4 acc = merged_o(hd, d4);
-            const float lh = merged_l(hd);
-            floatx4 o;
-#pragma unroll
-            for (int e = 0; e < 4; e++) {
-                o[e] = acc[e] / lh;
-            }
-            *reinterpret_cast<floatx4 *>(&a.out[(int64_t)(g * a.s.G + hd) * D + d4]) = o;
-        }
-        return;
-    }
-    // ---- the workgroup's partial, as 16-byte records that carry this launch's stamp in their first
-    // word: per head 32 records of four O values, cut to 24 bits each, and one of (max, sum).  A reader
-    // that sees the stamp has the whole record (a 16-byte store is performed as one), so the data is
-    // its own ready flag.
-    const unsigned int stamp32 = (unsigned int)(sh_gen + 1ull);
-    {
-        float *pw = a.part + ((int64_t)g * a.nsplit + split) * kDecodePartFloats;
-#pragma unroll
-        for (int it = 0; it < (16 * CHUNKS + P * 64 - 1) / (P * 64); it++) {
-            const int idx = tid + it * (P * 64);
-            if (idx < 16 * O_CHUNKS) {
-                const int hd = idx >> 5, ch = idx & 31;
-                if (hd < a.s.G) {
-                    st_dev4(pw + (hd * CHUNKS + ch) * 4, pack_record(stamp32, merged_o(hd, ch * 4)));
-                }
-            } else if (idx < 16 * CHUNKS) {
-                const int hd = idx - 16 * O_CHUNKS;
-                if (hd < a.s.G) {
-                    st_dev4(pw + (hd * CHUNKS + ML_CHUNK) * 4,
-                            uintx4{stamp32, __float_as_uint(sm_mwg[hd]), __float_as_uint(merged_l(hd)), 0u});
-                }
-            }
-        }
-    }
-
-    // ---- grid-wide merge.  Every workgroup merges one slice of the group's output from the partials
-    // of all splits, polling the records it needs until they carry this launch's stamp.  The poll is
-    // bounded: a workgroup whose wait runs out flags its slice as left behind and goes on to exit.
-    // Each workgroup also takes a ticket once its own partial is complete; the holder of the last
-    // ticket knows that every partial is complete, merges the slices it finds flagged, zeroes the
-    // ticket counter for the next launch and bumps the group's launch count.  Two workgroups may
-    // merge the same slice; they then write identical values.
-    //
-    // The last wave of the workgroup takes the ticket and waits for it (a trip to the device's
-    // coherence point, behind the tickets of the other workgroups).  The other waves merge without
-    // ever meeting that wave at a barrier.  The unit is a quad: four consecutive O records of one head
-    // (16 dims, 64 contiguous bytes of every split).  A quad is folded by 4 S lanes (s, rec): lane
-    // (s, rec) takes record rec of splits s, s + S, ... with a running max of its own, and the S lanes of
-    // a record are then merged.  With few splits (S <= 16) a wave holds 16 / S quads at a time and is on
-    // its own; with many, S = 32 or 64 lanes span 2 or 4 waves, whose results the first of them
-    // collects through LDS, in step with the others through LDS counters.
-    __shared__ int sh_last;
-    __shared__ int sh_flag;
-    __shared__ int sh_fail;
-    __shared__ int sh_list[kMaxSplits];
-    __shared__ int sh_count;
-    __shared__ __attribute__((aligned(16))) float red_o[2][kDecodeMaxWaves][4][4];
-    __shared__ float red_m[2][kDecodeMaxWaves][4];
-    __shared__ float red_l[2][kDecodeMaxWaves][4];
-    __shared__ int red_fail[2][kDecodeMaxWaves];
-    __shared__ int red_written[kDecodeMaxWaves];  // passes each wave has left in red_*
-    __shared__ int red_read[kDecodeMaxWaves];     // passes each collecting wave has taken out of red_*
-    unsigned int *ctr = a.sync_ctr + g;
-    unsigned long long *gen = a.sync_gen + g;
-    unsigned long long *claim = a.sync_claim + (int64_t)g * kMaxSplits;
-    const unsigned long long stamp = sh_gen + 1ull;
-
-    const int G = a.s.G;
-    const int total_quads = G * (O_CHUNKS / 4);
-    const int qps = (total_quads + a.nsplit - 1) / a.nsplit;  // quads per slice
-    constexpr int nwc = kDecodeMaxWaves;                       // waves that merge
-    int s_log = 0;  // S = 1 << s_log lanes per record, two splits each at a time
-    while (s_log < 6 && (2 << s_log) < a.nsplit) {
-        s_log++;
-    }
-    const int wpq_log = s_log > 4 ? s_log - 4 : 0;  // waves per quad: 1, 2 or 4
-    const int sw_log = s_log - wpq_log;             // lanes per record within one wave
-    const int wpq = 1 << wpq_log;
-    const int qpw = 16 >> sw_log;                   // quads per wave at a time
-    const int qpp = wpq > 1 ? nwc >> wpq_log : nwc * qpw;  // quads per pass of the workgroup
-    const float *part_g = a.part + (int64_t)g * a.nsplit * kDecodePartFloats;
-    int passes_done = 0;  // the same in every merging wave
-    if (tid < kDecodeMaxWaves) {
-        red_written[tid] = 0;
-        red_read[tid] = 0;
-    }
-    if (tid == 0) {
-        sh_fail = 0;
-    }
-
-    // Slice sl; called by the merging waves.  If the wait runs out the slice is abandoned and sh_fail set.
-    auto combine_slice = [&](int sl, unsigned long long t0, unsigned long long limit) {
-        const int q_begin = sl * qps;
-        const int q_end = (sl + 1) * qps < total_quads ? (sl + 1) * qps : total_quads;
-        const int rec4 = lane & 3, s_in_wave = (lane >> 2) & ((1 << sw_log) - 1), qslot = lane >> (2 + sw_log);
-        const int wq = w >> wpq_log, wsub = w & (wpq - 1);
-        const int s_lane = (wsub << sw_log) + s_in_wave;  // 0 .. S - 1
-        int failed = 0;
-        for (int q0 = q_begin; q0 < q_end; q0 += qpp, passes_done++) {
-            const int q = q0 + (wpq > 1 ? wq : w * qpw + qslot);
-            const bool valid = q < q_end;
-            const int qc = valid ? q : q_end - 1;
-            const int hl = qc >> 3, rec = (qc & 7) * 4 + rec4;
-            const float *obase = part_g + (hl * CHUNKS + rec) * 4;
-            const float *mbase = part_g + (hl * CHUNKS + ML_CHUNK) * 4;
-            Partial acc = {-INFINITY, 0.f, floatx4{0.f, 0.f, 0.f, 0.f}};
-            for (int b0 = 0; b0 < a.nsplit && !failed; b0 += 2 << s_log) {
-                const float *po[2], *pm[2];
-                bool ok[2];
-                uintx4 o4[2], ml4[2];
-                unsigned long long stale[2];
-#pragma unroll
-                for (int u = 0; u < 2; u++) {
-                    const int sp = b0 + (u << s_log) + s_lane;
-                    ok[u] = valid && sp < a.nsplit;
-                    const int spc = sp < a.nsplit ? sp : 0;
-                    po[u] = obase + (int64_t)spc * kDecodePartFloats;
-                    pm[u] = mbase + (int64_t)spc * kDecodePartFloats;
-                    o4[u] = uintx4{0u, 0u, 0u, 0u};
-                    ml4[u] = uintx4{0u, 0u, 0u, 0u};
-                    stale[u] = __ballot(ok[u]);
-                }
-                while (true) {
-                    ld_dev4x4(po, pm, o4, ml4, stale);  // only what has not arrived yet is loaded again
-#pragma unroll
-                    for (int u = 0; u < 2; u++) {
-                        const bool have = !ok[u] || (o4[u][0] == stamp32 && ml4[u][0] == stamp32);
-                        stale[u] = __ballot(!have);
-                    }
-                    if ((stale[0] | stale[1]) == 0ull) {
-                        break;
-                    }
-                    if (wall_clock64() - t0 > limit) {
-                        failed = 1;
-                        break;
-                    }
-                    __builtin_amdgcn_s_sleep(1);
-                }
-                if (!failed) {
-                    float mv[2];
-                    float m_new = acc.m;
-#pragma unroll
-                    for (int u = 0; u < 2; u++) {
-                        mv[u] = ok[u] ? __uint_as_float(ml4[u][1]) : -INFINITY;
-                        m_new = fmaxf(m_new, mv[u]);
-                    }
-                    if (m_new != -INFINITY) {
-                        const float sc = (acc.m == -INFINITY) ? 0.f : __expf(acc.m - m_new);
-                        acc.l *= sc;
-                        acc.o *= sc;
-#pragma unroll
-                        for (int u = 0; u < 2; u++) {
-                            const float fu = (mv[u] == -INFINITY) ? 0.f : __expf(mv[u] - m_new);
-                            const floatx4 ov = unpack_record(o4[u]);
-                            acc.l = __builtin_fmaf(fu, __uint_as_float(ml4[u][2]), acc.l);
-#pragma unroll
-                            for (int e = 0; e < 4; e++) {
-                                acc.o[e] = __builtin_fmaf(fu, ov[e], acc.o[e]);
-                            }
-                        }
-                        acc.m = m_new;
-                    }
-                }
-            }
-            if (failed) {
-                sh_fail = 1;
-            }
-            // the lanes of a record within the wave
-            bool writer;
-            if (sw_log == 4) {
-                // 16 lanes, 4 apart: 4 and 8 lanes down within each row of 16, then across the rows
-                acc = merge_partials(acc, row_shr<4>(acc));
-                acc = merge_partials(acc, row_shr<8>(acc));
-                acc = merge_partials(acc, lane_xor(acc, 16));
-                acc = merge_partials(acc, lane_xor(acc, 32));
-                writer = lane >= 12 && lane < 16;
-            } else {
-                if (sw_log > 0) acc = merge_partials(acc, lane_xor(acc, 4));
-                if (sw_log > 1) acc = merge_partials(acc, lane_xor(acc, 8));
-                if (sw_log > 2) acc = merge_partials(acc, lane_xor(acc, 16));
-                writer = s_in_wave == 0;
-            }
-            int bad = failed;  // a quad whose wait ran out anywhere is not written: whoever redoes the slice writes it
-            if (wpq > 1) {
-                // hand the wave's result to the first wave of the quad; red_* of this parity is free
-                // once that wave has collected the pass before the previous one
-                const int buf = passes_done & 1, lead = w & ~(wpq - 1);
-                if (w != lead) {
-                    while (*(volatile int *)&red_read[lead] < passes_done - 1) {
-                        __builtin_amdgcn_s_sleep(1);
-                    }
-                    if (writer) {
-                        red_m[buf][w][rec4] = acc.m;
-                        red_l[buf][w][rec4] = acc.l;
-                        *reinterpret_cast<floatx4 *>(&red_o[buf][w][rec4][0]) = acc.o;
-                    }
-                    if (lane == 0) {
-                        red_fail[buf][w] = failed;
-                    }
-                    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
-                    if (lane == 0) {
-                        *(volatile int *)&red_written[w] = passes_done + 1;
-                    }
-                    writer = false;
-                } else {
-                    while (!__all(lane == 0 || lane >= wpq || *(volatile int *)&red_written[lead + (lane & 3)] > passes_done)) {
-                        __builtin_amdgcn_s_sleep(1);
-                    }
-                    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
-                    for (int i = 1; i < wpq; i++) {
-                        bad |= red_fail[buf][lead + i];
-                    }
-                    if (writer) {
-                        Partial other[kDecodeMaxWaves];
-#pragma unroll
-                        for (int i = 1; i < kDecodeMaxWaves; i++) {  // rows past the quad's waves are read and dropped
-                            const int ww = (lead + i) & (kDecodeMaxWaves - 1);
-                            other[i].m = red_m[buf][ww][rec4];
-                            other[i].l = red_l[buf][ww][rec4];
-                            other[i].o = *reinterpret_cast<const floatx4 *>(&red_o[buf][ww][rec4][0]);
-                        }
-#pragma unroll
-                        for (int i = 1; i < kDecodeMaxWaves; i++) {
-                            if (i >= wpq) {
-                                other[i].m = -INFINITY;
-                                other[i].l = 0.f;
-                                other[i].o = floatx4{0.f, 0.f, 0.f, 0.f};
-                            }
-                            acc = merge_partials(acc, other[i]);
-                        }
-                    }
-                    if (lane == 0) {
-                        __hip_atomic_store(&red_read[lead], passes_done + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
-                    }
-                }
-            }
-            if (writer && valid && !bad) {
-                floatx4 o;
+            for (int T = 0; T < 4; T++) {
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
-                    o[e] = acc.o[e] / acc.l;
+                    if ((T >> 1) * 32 + c * 8 + (T & 1) * 4 + e >= limit) {
+                        s[T][e] = -INFINITY;
+                    }
                 }
-                *reinterpret_cast<floatx4 *>(&a.out[(int64_t)(g * G + hl) * D + rec * 4]) = o;
             }
         }
-    };
+        float mx = fmaxf(fmaxf(s[0][0], s[0][1]), fmaxf(s[0][2], s[0][3]));
+#pragma unroll
+        for (int T = 1; T < 4; T++) {
+            mx = fmaxf(mx, fmaxf(fmaxf(s[T][0], s[T][1]), fmaxf(s[T][2], s[T][3])));
+        }
+        mx = max_over_c(mx);
+        if (r == 0) {
+            mx = fmaxf(mx, s_new);
+        }
+        if (c == 0) {
+            sh.m[r & 1][w][j] = mx;
+        }
+        lds_signal(&sh.m_ready, lane);
+        TS(2);
+        lds_wait_ge(&sh.m_ready, W * (r + 1), a.flags);
+        float m_new = m_run;
+#pragma unroll
+        for (int ww = 0; ww < W; ww++) {
+            m_new = fmaxf(m_new, sh.m[r & 1][ww][j]);
+        }
+        const float m_ref = (m_new == -INFINITY) ? 0.f : m_new;  // no visible key yet: every p below is 0
+        const float alpha = (m_run == -INFINITY) ? 0.f : __expf(m_run - m_ref);
+        float psum = 0.f;
+        half8 pf[2];
+#pragma unroll
+        for (int T = 0; T < 4; T++) {
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const float pv = __expf(s[T][e] - m_ref);  // exp(-inf) = 0 for masked keys
+                psum += pv;
+                pf[T >> 1][(T & 1) * 4 + e] = (_Float16)pv;
+            }
+        }
+        psum = sum_over_c(psum);
+        float pn = 0.f;
+        if (r == 0 && s_new != -INFINITY) {
+            pn = (float)(_Float16)__expf(s_new - m_ref);
+            psum += pn;
+        }
+        l_run = l_run * alpha + psum;
+        m_run = m_new;
+        if (r > 0) {
+            lds_wait_ge(&sh.p_done, W * r, a.flags);  // the output waves are through with the last round's P
+        }
+        *reinterpret_cast<half8 *>(&sh.p[j][w * TILE + c * 8]) = pf[0];
+        *reinterpret_cast<half8 *>(&sh.p[j][w * TILE + 32 + c * 8]) = pf[1];
+        if (c == 0) {
+            sh.l[w][j] = l_run;
+            if (w == 0) {
+                sh.mrun[r & 1][j] = m_new;
+                if (r == 0) {
+                    sh.pnew[j] = pn;
+                }
+            }
+        }
+        lds_signal(&sh.p_ready, lane);
+    }
+    TS(3);
+}
 
-    wait_stores_dev();
-    __syncthreads();  // every partial store of this workgroup is complete before it takes its ticket
-    const bool mine = split * qps < total_quads;
-    if (w == nwc) {
-        if (lane == 0) {
-            const unsigned int ticket = __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            const bool last = (ticket == (unsigned int)a.nsplit - 1u);
-            if (last) {
-                __hip_atomic_store(ctr, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                __hip_atomic_store(gen, stamp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+// ---- output waves: O^T of 32 output dims over all keys of the workgroup.  Returns the lane's O (dims
+// w*32 + jb*16 + c*4 .. of head j), the head's sum and running max.
+__device__ inline void output_wave(const DecodeArgs &a, DecodeShared &sh, const Geom &ge, floatx4 (&o)[2],
+                                   float &l_tot, float &m_fin) {
+    const int lane = ge.lane, w = ge.w, j = ge.j, c = ge.c, g = ge.g;
+    const int L = a.s.L;
+    const __half *Vg = a.v_cache + (int64_t)g * D * L;
+
+    int nk = ge.te - ge.tb < W ? ge.te - ge.tb : W;
+    half8 vf[2][8];
+    load_v_dims<0, 8>(Vg, L, ge.tb * TILE, nk, w, lane, vf);
+    float vnew[2][4];
+    if (ge.owner_wg) {
+        // chatglm.cpp:672-675: v of the new token goes to the cache as fp16, and into this launch's output
+        const float *vhead = a.qkv + a.lay.v_off + (int64_t)g * a.lay.head_stride + w * 32;
+#pragma unroll
+        for (int jb = 0; jb < 2; jb++) {
+            const floatx4 vraw = *reinterpret_cast<const floatx4 *>(vhead + jb * 16 + c * 4);
+            _Float16 v16[4];
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                v16[e] = (_Float16)vraw[e];
+                vnew[jb][e] = (float)v16[e];
             }
-            sh_last = last;
-        }
-    } else if (mine) {
-        combine_slice(split, wall_clock64(), (unsigned long long)a.spin_ticks);
-    }
-    __syncthreads();
-    if (sh_fail) {
-        // Flag the slice for the holder of the last ticket, then look once more: if that workgroup
-        // is already past its scan, every partial is complete by now and this attempt succeeds.
-        // (The attempt starts after the flag is known to be in place.)
-        if (tid == 0) {
-            const unsigned long long old =
-                __hip_atomic_exchange(claim + split, stamp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            sh_flag = (old != ~0ull);
-        }
-        __syncthreads();
-        if (sh_flag && w < nwc) {
-            combine_slice(split, wall_clock64(), 0ull);
+            if (j < 4) {
+                const _Float16 mine = j == 0 ? v16[0] : j == 1 ? v16[1] : j == 2 ? v16[2] : v16[3];
+                *reinterpret_cast<_Float16 *>(a.v_cache + ((int64_t)g * D + w * 32 + jb * 16 + c * 4 + j) * L + a.p0) =
+                    mine;
+            }
         }
     }
-    if (!sh_last) {
+    TS(0);
+    o[0] = floatx4{0.f, 0.f, 0.f, 0.f};
+    o[1] = floatx4{0.f, 0.f, 0.f, 0.f};
+    float m_run = -INFINITY;
+    for (int r = 0; r < ge.rounds; r++) {
+        const int rt0 = ge.tb + r * W;
+        if (r > 0) {
+            nk = ge.te - rt0 < W ? ge.te - rt0 : W;
+            load_v_dims<0, 8>(Vg, L, rt0 * TILE, nk, w, lane, vf);
+        }
+        lds_wait_ge(&sh.p_ready, W * (r + 1), a.flags);
+        TS(3);
+        const float m_new = sh.mrun[r & 1][j];
+        const float alpha = (m_run == -INFINITY) ? 0.f : __expf(m_run - m_new);
+        m_run = m_new;
+        if ((rt0 + nk) * TILE > a.p0) {
+            // V columns of keys that do not exist may hold anything (never written, or stale): zero them
+#pragma unroll
+            for (int ks = 0; ks < 8; ks++) {
+                const int nv = a.p0 - (rt0 * TILE + ks * 32 + c * 8);  // keys of this lane's eight that exist
+                if (nv < 8) {
+#pragma unroll
+                    for (int jb = 0; jb < 2; jb++) {
+#pragma unroll
+                        for (int e = 0; e < 8; e++) {
+                            if (e >= nv) {
+                                vf[jb][ks][e] = (_Float16)0.f;
+                            }
+                        }
+                    }
+                }
+            }
+        }
+        o[0] *= alpha;
+        o[1] *= alpha;
+#pragma unroll
+        for (int ks = 0; ks < 8; ks++) {
+            if (ks < 2 * nk) {
+                const half8 pb = *reinterpret_cast<const half8 *>(&sh.p[j][ks * 32 + c * 8]);
+                o[0] = mfma16(vf[0][ks], pb, o[0]);
+                o[1] = mfma16(vf[1][ks], pb, o[1]);
+            }
+        }
+        if (r == 0 && ge.owner_wg) {
+            const float pn = sh.pnew[j];
+#pragma unroll
+            for (int jb = 0; jb < 2; jb++) {
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    o[jb][e] = __builtin_fmaf(pn, vnew[jb][e], o[jb][e]);
+                }
+            }
+        }
+        if (r + 1 < ge.rounds) {
+            lds_signal(&sh.p_done, lane);
+        }
+    }
+    // the sums of the score waves are each at the final running max
+    l_tot = 0.f;
+#pragma unroll
+    for (int ww = 0; ww < W; ww++) {
+        l_tot += sh.l[ww][j];
+    }
+    m_fin = m_run;
+    TS(4);
+}
+
+// Block = 8 waves: 4 score waves and 4 output waves, one of each per SIMD.  In a round the workgroup
+// takes up to 4 consecutive tiles (256 keys).  Score wave w loads the K rows of tile w and computes its
+// scores for all heads; the score waves agree on the maxes through LDS and leave their probabilities
+// there.  Output wave w meanwhile loads the V columns of output dims [32 w, 32 w + 32) for all keys of
+// the round (a wave that waits for room in the memory pipeline can do nothing else, which is why the two
+// kinds of work are in different waves) and then accumulates those dims over all keys.  O never goes
+// through LDS and ends up in the lanes in exactly the layout of the lines.
+template <int TYPE>
+__device__ inline void decode_body(const DecodeArgs &a, DecodeShared &sh) {
+    Geom ge;
+    ge.lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    ge.w = wave & (W - 1);
+    const bool scores = wave < W;
+    ge.t_start = wall_clock64();
+    TS(10);
+    ge.j = ge.lane & 15;
+    ge.c = ge.lane >> 4;
+    ge.g = blockIdx.y;
+    ge.split = blockIdx.x;
+    const int lane = ge.lane, w = ge.w, j = ge.j, c = ge.c, g = ge.g, split = ge.split;
+    const int G = a.s.G;
+    // tiles [tb, te) of the keys already in the cache are this workgroup's
+    ge.tb = split * a.tiles_q + (split < a.tiles_r ? split : a.tiles_r);
+    ge.te = ge.tb + a.tiles_q + (split < a.tiles_r ? 1 : 0);
+    ge.rounds = ge.te - ge.tb > W ? (ge.te - ge.tb + W - 1) / W : 1;
+    ge.owner_wg = split == a.nsplit - 1;  // appends the new token and attends to it
+
+    // The launch count stamps this launch's lines.  Every lane reads it (no branch, one request per
+    // wave) among its first loads: no workgroup can have finished before that.
+    const unsigned long long gen = __hip_atomic_load(&a.sync[g].gen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const unsigned int stamp32 = decode_stamp(gen);
+
+    const int total_quads = G * QUADS;
+    const int qps = (total_quads + a.nsplit - 1) / a.nsplit;  // quads per slice
+    MergeGeom mg;
+    mg.nsplit = a.nsplit;
+    mg.G = G;
+    mg.sl_log = 0;
+    while (mg.sl_log < 4 && (1 << mg.sl_log) < a.nsplit) {
+        mg.sl_log++;
+    }
+    mg.stamp32 = stamp32;
+    mg.part_g = a.part + (int64_t)g * a.nsplit * kDecodePartFloats;
+    mg.out_g = a.out + (int64_t)g * G * D;
+    DecodeGroupSync *sy = a.sync + g;
+    unsigned long long *claim = a.claim + (int64_t)g * kDecodeMaxSplits;
+    const unsigned long long stamp = gen + 1ull;
+
+    if (scores) {
+        score_wave<TYPE>(a, sh, ge);
+        if (a.nsplit == 1) {
+            return;
+        }
+        // ---- grid-wide merge.  The score waves of every workgroup fold the quads of one slice of the
+        // group's output from the lines of all splits, which they load past the caches and poll until
+        // they carry this launch's stamp.  The poll is bounded: a wave whose wait runs out flags the
+        // slice as left behind, looks once more and goes on to exit.  An output wave takes a ticket
+        // once the lines of the whole workgroup have been performed; the holder of the last ticket
+        // knows that every partial is complete, merges the slices it finds flagged, zeroes the ticket
+        // counter for the next launch and bumps the launch count.  Two waves may merge the same slice;
+        // they then write identical values.
+        const int q_begin = split * qps;
+        const int q_end = (split + 1) * qps < total_quads ? (split + 1) * qps : total_quads;
+        const int qw = 16 >> mg.sl_log;
+        if (q_begin + w * qw >= q_end) {
+            return;
+        }
+        const unsigned long long t0 = wall_clock64();
+        const unsigned long long limit = (unsigned long long)a.spin_ticks;
+        // The lines are polled directly (a shared arrival counter would be one hot address for all the
+        // workgroups of a group).  Other workgroups finish up to a good fraction of this one's own run
+        // time later, and a line takes a while to become visible: looking right away would load nearly
+        // every line twice, so the first look waits a little.
+        {
+            const unsigned long long wait_ticks = (t0 - ge.t_start) / EXP_DELAY_DIV + EXP_DELAY_ADD;
+            while (wall_clock64() - t0 < wait_ticks && wait_ticks < limit) {
+                __builtin_amdgcn_s_sleep(4);
+            }
+        }
+        TS(6);
+        int failed = merge_quads(mg, q_begin, q_end, w, W, lane, t0, limit);
+        TS(7);
+        if (failed) {
+            // Flag the slice for the holder of the last ticket (the slice's word, then a count in the
+            // ticket word, which that workgroup sees in the answer to its own ticket), then look once
+            // more: if that workgroup already has its ticket, every partial is complete by now and
+            // this attempt succeeds.  (The attempt starts after both are known to be in place.)
+            if (lane == 0) {
+                (void)__hip_atomic_exchange(claim + split, stamp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                (void)__hip_atomic_fetch_add(&sy->ticket, 0x10000u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+            wait_vm();
+            (void)merge_quads(mg, q_begin, q_end, w, W, lane, wall_clock64(), 0ull);
+        }
         return;
     }
-    // slices whose owners left: normally none
-    if (tid == 0) {
-        sh_count = 0;
+
+    floatx4 o[2];
+    float l_tot, m_fin;
+    output_wave(a, sh, ge, o, l_tot, m_fin);
+    if (a.nsplit == 1) {
+        // a single workgroup saw every key of the group: normalise and finish
+        if (j < G) {
+#pragma unroll
+            for (int jb = 0; jb < 2; jb++) {
+                floatx4 ov;
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    ov[e] = o[jb][e] / l_tot;
+                }
+                *reinterpret_cast<floatx4 *>(&a.out[(int64_t)(g * G + j) * D + w * 32 + jb * 16 + c * 4]) = ov;
+            }
+        }
+        return;
     }
-    __syncthreads();
-    for (int sl = tid; sl < a.nsplit; sl += blockDim.x) {
-        if (sl * qps < total_quads &&
-            __hip_atomic_load(claim + sl, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == stamp) {
-            sh_list[atomicAdd(&sh_count, 1)] = sl;
+    // ---- the workgroup's partial as stamped lines: O / sum and max + ln(sum) per head.  Lane (j, c)
+    // of output wave w holds piece c of quads 2 w and 2 w + 1 of head j.
+    if (j < G) {
+        float *pw = a.part + ((int64_t)g * a.nsplit + split) * kDecodePartFloats;
+        const float inv = l_tot > 0.f ? __builtin_amdgcn_rcpf(l_tot) : 0.f;
+        const unsigned int lse = __float_as_uint(l_tot > 0.f ? m_fin + __logf(l_tot) : -INFINITY);
+#pragma unroll
+        for (int jb = 0; jb < 2; jb++) {
+            st_dev4(pw + ((j * QUADS + w * 2 + jb) * 4 + c) * 4, pack_piece(stamp32, o[jb] * inv, lse, c));
         }
     }
-    __syncthreads();
-    const int n_left = sh_count;
-    const unsigned long long sweep_limit = a.spin_ticks > 10000 ? (unsigned long long)a.spin_ticks : 10000ull;
-    if (w < nwc) {
-        for (int i = 0; i < n_left; i++) {
-            combine_slice(sh_list[i], wall_clock64(), sweep_limit);
+    TS(5);
+    // ---- ticket, and the sweep if this workgroup holds the last one
+    wait_vm();  // this wave's line stores have been performed
+    lds_signal(&sh.stored, lane);
+    if (w != 0) {
+        return;
+    }
+    lds_wait_ge(&sh.stored, W, a.flags);
+    unsigned int ticket = 0;
+    if (lane == 0) {
+        ticket = __hip_atomic_fetch_add(&sy->ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    ticket = __shfl(ticket, 0);
+    if ((ticket & 0xffffu) != (unsigned int)a.nsplit - 1u) {
+        return;
+    }
+    TS(8);
+    // slices whose owners left before this ticket: normally none, and then nothing is scanned
+    if (ticket >> 16) {
+        const unsigned long long sweep_limit = a.spin_ticks > 10000 ? (unsigned long long)a.spin_ticks : 10000ull;
+        const int n_slices = (total_quads + qps - 1) / qps;
+        int lost = 0;
+        for (int sl0 = 0; sl0 < n_slices; sl0 += 64) {
+            unsigned long long cl = 0;
+            if (sl0 + lane < n_slices) {
+                cl = __hip_atomic_load(claim + sl0 + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+            unsigned long long left = __ballot(sl0 + lane < n_slices && cl == stamp);
+            while (left) {
+                const int sl = sl0 + __builtin_ctzll(left);
+                left &= left - 1;
+                const int qb = sl * qps;
+                const int qe = (sl + 1) * qps < total_quads ? (sl + 1) * qps : total_quads;
+                lost |= merge_quads(mg, qb, qe, 0, 1, lane, wall_clock64(), sweep_limit);
+            }
         }
+        if (lost && lane == 0) {
+            atomicOr(a.flags, kFlagMergeIncomplete);
+        }
+    }
+    // the launch is over for this group: words for the next one
+    if (lane == 0) {
+        __hip_atomic_store(&sy->ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(&sy->gen, decode_next_gen(gen), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    TS(9);
+}
+
+__global__ __launch_bounds__(kBlock) void decode_kernel(DecodeArgs a) {
+    __shared__ DecodeShared sh;
+    if (threadIdx.x == 0) {
+        sh.m_ready = 0;
+        sh.p_ready = 0;
+        sh.p_done = 0;
+        sh.stored = 0;
+    }
+    __syncthreads();
+    switch (a.rope.pairs > 0 ? a.rope.type : GLM_ATTN_ROPE_DISABLED) {
+    case GLM_ATTN_ROPE_GPTJ:
+        decode_body<GLM_ATTN_ROPE_GPTJ>(a, sh);
+        break;
+    case GLM_ATTN_ROPE_NEOX:
+        decode_body<GLM_ATTN_ROPE_NEOX>(a, sh);
+        break;
+    case GLM_ATTN_ROPE_CHATGLM:
+        decode_body<GLM_ATTN_ROPE_CHATGLM>(a, sh);
+        break;
+    case GLM_ATTN_ROPE_CHATGLM2:
+        decode_body<GLM_ATTN_ROPE_CHATGLM2>(a, sh);
+        break;
+    default:
+        decode_body<GLM_ATTN_ROPE_DISABLED>(a, sh);
+        break;
     }
 }
 
 }  // namespace
 
+#ifdef GLM_ATTN_TIMELINE
+// Only in the instrumented build: copies the clock readings of the last decode launch to the host.
+extern "C" int glm_attn_debug_decode_timeline(unsigned long long *host, size_t n) {
+    if (n > (size_t)kTimelineSlots * 16) n = (size_t)kTimelineSlots * 16;
+    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(g_decode_timeline), n * sizeof(unsigned long long));
+}
+#endif
+
 hipError_t launch_decode(const DecodeArgs &a, hipStream_t stream) {
-    if (a.nsplit < 1 || a.nsplit > kMaxSplits || a.waves < 1 || a.waves > kDecodeMaxWaves) {
+    if (a.nsplit < 1 || a.nsplit > kDecodeMaxSplits || a.tiles_q < 0 || a.tiles_r < 0 || a.tiles_r >= a.nsplit) {
         return hipErrorInvalidValue;
     }
-    // always the full block: waves without keys to read still take part in the merges
-    hipLaunchKernelGGL(decode_kernel, dim3(a.nsplit, a.s.kvh), dim3((kDecodeMaxWaves + 1) * 64), 0, stream, a);
+    hipLaunchKernelGGL(decode_kernel, dim3(a.nsplit, a.s.kvh), dim3(kBlock), 0, stream, a);
     return hipGetLastError();
 }
 
 }  // namespace glm_attn
-

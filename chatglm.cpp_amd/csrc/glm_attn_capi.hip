@@ -32,9 +32,8 @@ struct glm_attn_ctx {
     int64_t prefill_floats;
     int max_splits;
     void *sync_mem;      // hand-over words of the decode kernel (see DecodeArgs)
-    unsigned int *sync_ctr;
-    unsigned long long *sync_gen;
-    unsigned long long *sync_claim;
+    DecodeGroupSync *sync;
+    unsigned long long *claim;
     long long spin_ticks;
     uint32_t *flags;
     int last_hip_error;
@@ -238,24 +237,21 @@ int do_decode(glm_attn_ctx *c, int layer, const float *qkv, const int32_t *posit
     da.scale = c->scale;
     da.k_cache = layer_k(c, layer);
     da.v_cache = layer_v(c, layer);
-    // Deal the 64-key tiles of a group out to as many workgroups as there are CUs for it, then to
-    // up to 4 waves per workgroup: spreading over CUs first buys more load queues.
+    // Deal the 64-key tiles of a group out to as many workgroups as there are CUs for it: spreading
+    // over CUs first buys more load queues.  A workgroup takes its tiles four at a time.
     const int n_tiles = (da.p0 + kDecodeTileKeys - 1) / kDecodeTileKeys;
     const int cu_share = c->num_cus / c->shape.kvh > 0 ? c->num_cus / c->shape.kvh : 1;
-    int wpg = n_tiles < 1 ? 1 : n_tiles;
-    if (wpg > kDecodeMaxWaves * cu_share) wpg = kDecodeMaxWaves * cu_share;
-    int nsplit = wpg < cu_share ? wpg : cu_share;
+    int nsplit = n_tiles < 1 ? 1 : n_tiles;
+    if (nsplit > cu_share) nsplit = cu_share;
     if (nsplit > c->max_splits) nsplit = c->max_splits;
-    int waves = (wpg + nsplit - 1) / nsplit;
-    if (waves > kDecodeMaxWaves) waves = kDecodeMaxWaves;
     da.nsplit = nsplit;
-    da.waves = waves;
+    da.tiles_q = n_tiles / nsplit;
+    da.tiles_r = n_tiles % nsplit;
     da.part = c->part;
     da.out = out;
     da.flags = c->flags;
-    da.sync_ctr = c->sync_ctr;
-    da.sync_gen = c->sync_gen;
-    da.sync_claim = c->sync_claim;
+    da.sync = c->sync;
+    da.claim = c->claim;
     da.spin_ticks = c->spin_ticks;
     HIP_TRY(c, launch_decode(da, stream));
     return GLM_ATTN_OK;
@@ -396,18 +392,16 @@ int glm_attn_create(const glm_attn_desc *desc, glm_attn_ctx **out_ctx) {
     c->max_splits = c->num_cus / s.kvh > 0 ? c->num_cus / s.kvh : 1;
     if (c->max_splits > kDecodeMaxSplits) c->max_splits = kDecodeMaxSplits;
     {
-        // [kvh] launch counts (u64), [kvh][kDecodeMaxSplits] claims (u64), [kvh][2] arrival counters (u32)
-        const size_t n64 = (size_t)s.kvh * (1 + kDecodeMaxSplits);
-        const size_t bytes = n64 * sizeof(unsigned long long) + 2 * (size_t)s.kvh * sizeof(unsigned int);
+        // [kvh] counters, then [kvh][kDecodeMaxSplits] claims (u64)
+        const size_t bytes = (size_t)s.kvh * (sizeof(DecodeGroupSync) + kDecodeMaxSplits * sizeof(unsigned long long));
         CREATE_TRY(hipMalloc(&c->sync_mem, bytes));
         CREATE_TRY(hipMemset(c->sync_mem, 0, bytes));
-        c->sync_gen = static_cast<unsigned long long *>(c->sync_mem);
-        c->sync_claim = c->sync_gen + s.kvh;
-        c->sync_ctr = reinterpret_cast<unsigned int *>(c->sync_claim + (size_t)s.kvh * kDecodeMaxSplits);
+        c->sync = static_cast<DecodeGroupSync *>(c->sync_mem);
+        c->claim = reinterpret_cast<unsigned long long *>(c->sync + s.kvh);
         c->spin_ticks = 100 * 100;  // 100 us at the 100 MHz constant clock
     }
     {
-        // the records of the partials carry launch stamps, which start at 1: begin with none that matches
+        // the lines of the partials carry launch stamps, which are never 0: begin with none that matches
         const size_t bytes = sizeof(float) * (size_t)s.kvh * c->max_splits * kDecodePartFloats;
         CREATE_TRY(hipMalloc((void **)&c->part, bytes));
         CREATE_TRY(hipMemset(c->part, 0, bytes));

@@ -20,9 +20,30 @@ constexpr int kMaxGroupHeads = 16;   // q heads of one KV group fill the 16 colu
 constexpr int kDecodeTileKeys = 64;  // keys one wave consumes per step of the decode kernel
 constexpr int kDecodeMaxWaves = 4;   // tile waves per workgroup of the decode kernel
 constexpr int kDecodeMaxSplits = 512;  // workgroups per KV group of the decode kernel
-// floats of one (group, split) partial of the decode kernel: 16 heads x 33 records of 16 bytes
-constexpr int kDecodePartFloats = 16 * 33 * 4;
+// floats of one (group, split) partial of the decode kernel: 16 heads x 8 lines of 64 bytes
+constexpr int kDecodePartFloats = 16 * 8 * 16;
+constexpr int kDecodeHintShards = 4;   // arrival counters per KV group, one 64-byte line each
+constexpr int kTimelineSlots = 4096;   // waves recorded by the instrumented build of the decode kernel
 constexpr uint32_t kFlagPositionClamped = 1u;
+constexpr uint32_t kFlagMergeIncomplete = 2u;  // a slice of a decode output was left unwritten
+
+// Hand-over words of the decode kernel, one set per KV group.
+struct DecodeGroupSync {
+    unsigned long long gen;   // launches of this group completed so far (with more than one split)
+    unsigned int hint_base;   // sum of the hint counters when the current launch began
+    unsigned int ticket;      // low 16 bits: workgroups whose lines are performed; above: slices left behind
+    unsigned int pad[12];
+    unsigned int hint[kDecodeHintShards][16];  // workgroups that have issued their lines, ever (word 0 of each line)
+};
+static_assert(sizeof(DecodeGroupSync) == 64 * (1 + kDecodeHintShards), "one line per counter");
+
+// The 32-bit stamp of the lines written by the launch that follows `gen` completed ones.  It is never
+// 0 (what a zero-filled exchange buffer holds): decode_next_gen skips the count whose stamp would be.
+__host__ __device__ inline unsigned int decode_stamp(unsigned long long gen) { return (unsigned int)(gen + 1ull); }
+__host__ __device__ inline unsigned long long decode_next_gen(unsigned long long gen) {
+    const unsigned long long next = gen + 1ull;
+    return decode_stamp(next) == 0u ? next + 1ull : next;
+}
 
 // Where q, k and v heads sit inside one token's row of the fused projection (chatglm.cpp:636-653).
 struct QkvLayout {
@@ -84,15 +105,14 @@ struct DecodeArgs {
     __half *k_cache;
     __half *v_cache;
     int nsplit;     // workgroups per KV group
-    int waves;      // waves per workgroup
-    float *part;    // [kvh][nsplit][kDecodePartFloats] split partials as stamped 16-byte records
+    int tiles_q, tiles_r;  // tiles of 64 cached keys per workgroup: tiles_q, one more in the first tiles_r
+    float *part;    // [kvh][nsplit][kDecodePartFloats] split partials as stamped 64-byte lines
     float *out;     // [h d]
     uint32_t *flags;
-    // grid-wide hand-over of the split partials (one set per KV group)
-    unsigned int *sync_ctr;         // [kvh] arrivals of the current launch, back to 0 when it ends
-    unsigned long long *sync_gen;   // [kvh] launches completed so far
-    unsigned long long *sync_claim; // [kvh][kDecodeMaxSplits] stamp of the launch that last left each slice behind
-    long long spin_ticks;           // bound on the wait for the other workgroups, in 100 MHz ticks
+    // grid-wide hand-over of the split partials
+    DecodeGroupSync *sync;      // [kvh]
+    unsigned long long *claim;  // [kvh][kDecodeMaxSplits] launch (gen + 1) that last left each slice behind
+    long long spin_ticks;       // bound on the wait for the other workgroups, in 100 MHz ticks
 };
 
 // activations of BasicMLP / BasicGLU (chatglm.cpp:444-454), shared by the elementwise kernel and the fused Linear
