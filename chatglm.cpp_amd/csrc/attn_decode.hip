@@ -29,9 +29,17 @@ __device__ unsigned long long g_decode_timeline[kTimelineSlots * 16];
         const int slot_ = (blockIdx.y * gridDim.x + blockIdx.x) * 2 * kDecodeMaxWaves + (threadIdx.x >> 6);      \
         if ((threadIdx.x & 63) == 0 && slot_ < kTimelineSlots) g_decode_timeline[slot_ * 16 + (i)] = wall_clock64(); \
     } while (0)
+#define TSCOUNT(i)                                                                                           \
+    do {                                                                                                     \
+        const int slot_ = (blockIdx.y * gridDim.x + blockIdx.x) * 2 * kDecodeMaxWaves + (threadIdx.x >> 6);  \
+        if ((threadIdx.x & 63) == 0 && slot_ < kTimelineSlots) g_decode_timeline[slot_ * 16 + (i)] += 1;      \
+    } while (0)
 #else
 #define TS(i) \
     do {      \
+    } while (0)
+#define TSCOUNT(i) \
+    do {           \
     } while (0)
 #endif
 
@@ -48,8 +56,8 @@ typedef unsigned int uintx4 __attribute__((ext_vector_type(4)));
 // ---------------------------------------------------------------------------------------------------
 // Lines of a split partial.  A line is four 16-byte pieces; piece p holds the launch's stamp, four
 // values of O / sum cut to 22 bits (sign, exponent, 13 mantissa bits, rounded to nearest: 2^-14
-// relative on values that are averages of V) and byte p of the fp32 log-sum-exp max + ln(sum) of the
-// (split, head).  A 16-byte store is performed as one, so a piece that shows the stamp is complete:
+// relative on values that are averages of V) and byte p of the fp32 base-2 log-sum-exp
+// max * log2(e) + log2(sum) of the (split, head).  A 16-byte store is performed as one, so a piece that shows the stamp is complete:
 // the data is its own ready flag.
 __device__ inline unsigned int round22(float x) {
     const unsigned int u = __float_as_uint(x);
@@ -232,121 +240,254 @@ __device__ inline void finish_row(const RowRegs &r, float scale, bool zero, half
 }
 
 // ---------------------------------------------------------------------------------------------------
+// The group's queries for the score waves: score wave w ropes, scales and rounds heads 4w .. 4w + 3
+// (lane: head 4w + (lane >> 4), dims (lane & 15) * 8 .. + 7) and leaves them in LDS, where all four
+// waves then pick up the whole operand.  Partners that are not among the lane's own eight dims (the
+// NEOX pairings) are simply loaded as well.
+constexpr int QPAD = D + 8;  // row pitch of the fp16 query tile in LDS (halfs): conflict-free b128 reads
+
+struct QPart {
+    floatx4 x[2], xp[2];
+    floatx4 cs[4];
+};
+
+template <int TYPE>
+__device__ inline void issue_q_part(const float *head, int d0, const int (&pos)[2], const RopeSpec &rope, QPart &r) {
+    r.x[0] = *reinterpret_cast<const floatx4 *>(head + d0);
+    r.x[1] = *reinterpret_cast<const floatx4 *>(head + d0 + 4);
+    if (TYPE == GLM_ATTN_ROPE_GPTJ || TYPE == GLM_ATTN_ROPE_CHATGLM2) {
+        // pair of dim d is d >> 1: four pairs from d0 / 2 (dims that are not rotated read the last four)
+        int p0 = d0 >> 1;
+        p0 = p0 <= rope.pairs - 4 ? p0 : rope.pairs - 4;
+        const float2 *row = rope.table + (int64_t)pos[0] * rope.pairs + p0;
+        r.cs[0] = *reinterpret_cast<const floatx4 *>(row);
+        r.cs[1] = *reinterpret_cast<const floatx4 *>(row + 2);
+    } else if (TYPE == GLM_ATTN_ROPE_NEOX) {
+        // pairs (d, d + 64), pair index d % 64
+        r.xp[0] = *reinterpret_cast<const floatx4 *>(head + (d0 ^ 64));
+        r.xp[1] = *reinterpret_cast<const floatx4 *>(head + (d0 ^ 64) + 4);
+        const float2 *row = rope.table + (int64_t)pos[0] * rope.pairs + (d0 & 63);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            r.cs[i] = *reinterpret_cast<const floatx4 *>(row + i * 2);
+        }
+    } else if (TYPE == GLM_ATTN_ROPE_CHATGLM) {
+        // NEOX inside each half of the head: pairs (el, el + 32), pair index el % 32, positions per half
+        r.xp[0] = *reinterpret_cast<const floatx4 *>(head + (d0 ^ 32));
+        r.xp[1] = *reinterpret_cast<const floatx4 *>(head + (d0 ^ 32) + 4);
+        const float2 *row = rope.table + (int64_t)pos[d0 >> 6] * rope.pairs + (d0 & 31);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            r.cs[i] = *reinterpret_cast<const floatx4 *>(row + i * 2);
+        }
+    }
+}
+
+// rope (chatglm.cpp:523-618), then `* scale` in fp32 (chatglm.cpp:686) and the fp16 rounding of ggml's
+// mat-mul operand
+template <int TYPE>
+__device__ inline half8 finish_q_part(const QPart &r, int d0, float scale, bool zero) {
+    half8 out;
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+        const float self = r.x[e >> 2][e & 3];
+        float x = self;
+        if (TYPE == GLM_ATTN_ROPE_GPTJ || TYPE == GLM_ATTN_ROPE_CHATGLM2) {
+            const float partner = r.x[e >> 2][(e & 3) ^ 1];
+            const floatx4 cs = r.cs[e >> 2];
+            const int k = (e >> 1) & 1;
+            const float xr = rope_rotate(self, partner, cs[2 * k], cs[2 * k + 1], !(e & 1));
+            x = (TYPE == GLM_ATTN_ROPE_GPTJ || d0 < D / 2) ? xr : self;
+        } else if (TYPE == GLM_ATTN_ROPE_NEOX) {
+            const floatx4 cs = r.cs[e >> 1];
+            x = rope_rotate(self, r.xp[e >> 2][e & 3], cs[2 * (e & 1)], cs[2 * (e & 1) + 1], d0 < 64);
+        } else if (TYPE == GLM_ATTN_ROPE_CHATGLM) {
+            const floatx4 cs = r.cs[e >> 1];
+            x = rope_rotate(self, r.xp[e >> 2][e & 3], cs[2 * (e & 1)], cs[2 * (e & 1) + 1], (d0 & 63) < 32);
+        }
+        out[e] = zero ? (_Float16)0.f : (_Float16)__fmul_rn(x, scale);
+    }
+    return out;
+}
+
+// ---------------------------------------------------------------------------------------------------
 // Merge across workgroups: fold the lines of all splits for quads [q_begin, q_end) of KV group g.
 // Quads are dealt out to the calling waves (wave `wi` of `nw`), `qw` of them at a time per wave: lane
 // (qslot, s, piece) takes piece `piece` of the lines of splits s, s + SL, ... of its quad.
 struct MergeGeom {
     int nsplit, G, sl_log;  // SL = 1 << sl_log lanes per (quad, piece)
     unsigned int stamp32;
-    const float *part_g;    // lines of the group: [nsplit][16 heads][QUADS][16 floats]
+    const float *part_g;    // lines of the group: [16 heads][QUADS][nsplit][16 floats], a slice's lines side by side
     float *out_g;           // [G][D]
+    unsigned long long *gen_word;  // the group's launch count, and what it becomes when this launch is over
+    unsigned long long gen_next;
 };
 
-// All-lanes reductions over the lanes that differ in bits [2, 2 + sl_log) of the lane index.  With 16
-// such lanes (the long-context shape) they need no LDS: two rotations inside the rows of 16 lanes fused
-// into the operation (DPP), then the two row swaps of gfx950.
+// All-lanes reductions over the lanes that differ in the upper sl_log bits of the lane index, without
+// LDS: the two row swaps of gfx950 for bits 5 and 4, rotations inside the rows of 16 lanes fused into
+// the operation (DPP) for bits 3 and 2 (a rotation by 8 pairs lanes 8 apart; with all four bits in
+// play, rotations by 4 and then 8 cover the four lanes 4 apart).
 __device__ inline float rot_row(float x, int n) {
     return n == 4 ? __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x124, 0xf, 0xf, false))
                   : __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x128, 0xf, 0xf, false));
 }
 template <typename F>
 __device__ inline float reduce_splits(float x, int sl_log, F op) {
-    if (sl_log == 4) {
-        x = op(x, rot_row(x, 4));
-        x = op(x, rot_row(x, 8));
+    if (sl_log > 3) x = op(x, rot_row(x, 4));
+    if (sl_log > 2) x = op(x, rot_row(x, 8));
+    if (sl_log > 1) {
         auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
         x = op(__uint_as_float(a[0]), __uint_as_float(a[1]));
-        auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
-        return op(__uint_as_float(b[0]), __uint_as_float(b[1]));
     }
-    if (sl_log > 0) x = op(x, __shfl_xor(x, 4));
-    if (sl_log > 1) x = op(x, __shfl_xor(x, 8));
-    if (sl_log > 2) x = op(x, __shfl_xor(x, 16));
+    if (sl_log > 0) {
+        auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+        x = op(__uint_as_float(b[0]), __uint_as_float(b[1]));
+    }
     return x;
 }
 
-// Returns 0 when every quad was written, 1 when the wait ran out (nothing is written for that pass).
+// One round of a poll: the lines that have shown up since the last round are folded into the lane's
+// running (max, sum, O), so that what is left to do after the last line has arrived is that line and the
+// reduction over the lanes.  A line counts when all four of its pieces carry the stamp (its log-sum-exp
+// is spread over them).  `want` has a bit per line this lane still needs; returns the lanes' union.
+struct Fold {
+    float m, w;
+    floatx4 o;
+};
+__device__ inline unsigned long long fold_round(const uintx4 (&r)[8], unsigned int &want, unsigned int stamp32,
+                                                int piece, unsigned long long (&pending)[8], Fold &acc) {
+    // which lines are new, and the base-2 log-sum-exp of each from the bytes in its four pieces
+    float lse[8];
+    float m_new = acc.m;
+    unsigned int got = 0;
+#pragma unroll
+    for (int it = 0; it < 8; it++) {
+        lse[it] = -INFINITY;
+        if (pending[it] == 0ull) {
+            continue;
+        }
+        int ok = ((want >> it) & 1u) && r[it][0] == stamp32;
+        ok &= __builtin_amdgcn_update_dpp(0, ok, 0xB1, 0xf, 0xf, true);  // quad_perm [1,0,3,2]
+        ok &= __builtin_amdgcn_update_dpp(0, ok, 0x4E, 0xf, 0xf, true);  // quad_perm [2,3,0,1]
+        int bits = (int)(r[it][3] >> 24) << (8 * piece);
+        bits |= __builtin_amdgcn_update_dpp(0, bits, 0xB1, 0xf, 0xf, true);
+        bits |= __builtin_amdgcn_update_dpp(0, bits, 0x4E, 0xf, 0xf, true);
+        if (ok) {
+            got |= 1u << it;
+            lse[it] = __int_as_float(bits);
+            m_new = fmaxf(m_new, lse[it]);
+        }
+    }
+    want &= ~got;
+    if (m_new != -INFINITY) {
+        const float sc = __builtin_amdgcn_exp2f(acc.m - m_new);  // exp2(-inf) = 0 for the first lines
+        acc.w *= sc;
+        acc.o *= sc;
+        acc.m = m_new;
+#pragma unroll
+        for (int it = 0; it < 8; it++) {
+            if (pending[it] == 0ull) {
+                continue;
+            }
+            const float wgt = __builtin_amdgcn_exp2f(lse[it] - m_new);  // 0 for lines that are not new
+            const floatx4 v = unpack_piece(r[it]);
+            acc.w += wgt;
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                acc.o[e] = __builtin_fmaf(wgt, v[e], acc.o[e]);
+            }
+        }
+    }
+    unsigned long long any = 0ull;
+#pragma unroll
+    for (int it = 0; it < 8; it++) {
+        if (pending[it] != 0ull) {
+            pending[it] = __ballot((want >> it) & 1u);
+            any |= pending[it];
+        }
+    }
+    return any;
+}
+
+// Polls and folds lines `first + it * step` (it = 0 .. 7, those below nsplit) of one (quad, piece) until
+// all have arrived.  Returns 1 when the wait ran out.
+__device__ inline int poll_lines(const float *base, int first, int step, int nsplit, bool valid, unsigned int stamp32,
+                                 int piece, unsigned long long t0, unsigned long long limit, Fold &acc) {
+    uintx4 r[8];
+    const float *p[8];
+    unsigned int want = 0;  // bit it: this lane still needs line it
+    unsigned long long pending[8];
+#pragma unroll
+    for (int it = 0; it < 8; it++) {
+        const int sp = first + it * step;
+        r[it] = uintx4{0u, 0u, 0u, 0u};
+        const bool need = valid && sp < nsplit;
+        want |= need ? 1u << it : 0u;
+        p[it] = base + (sp < nsplit ? sp : 0) * 16;
+        pending[it] = __ballot(need);
+    }
+    TS(13);
+    while (true) {
+        const unsigned long long now = wall_clock64();  // read while the loads are on their way
+        ld_lines8(p, r, pending);                       // only what has not arrived yet is loaded again
+        TSCOUNT(14);
+        TS(15);
+        const unsigned long long any = fold_round(r, want, stamp32, piece, pending, acc);
+        TS(12);
+        if (any == 0ull) {
+            return 0;
+        }
+        if (now - t0 > limit) {
+            return 1;
+        }
+        __builtin_amdgcn_s_sleep(1);
+    }
+}
+
+// What ends a slice: the (max, sum, O) of all lanes of a piece merged, normalised and stored.
+__device__ inline void reduce_fold(Fold &acc, int sl_log) {
+    const float m_all = reduce_splits(acc.m, sl_log, [](float x, float y) { return fmaxf(x, y); });
+    const float f = (acc.m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(acc.m - m_all);
+    auto add = [](float x, float y) { return x + y; };
+    acc.m = m_all;
+    acc.w = reduce_splits(acc.w * f, sl_log, add);
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        acc.o[e] = reduce_splits(acc.o[e] * f, sl_log, add);
+    }
+}
+
+// Merges quads [q_begin, q_end) of KV group g, dealt out to the calling waves (wave `wi` of `nw`), `qw`
+// of them at a time per wave: lane (s, quad of the pass, piece) takes piece `piece` of the lines of
+// splits s, s + SL, ... of its quad.  Returns 0 when every quad was written, 1 when the wait ran out
+// (nothing is written for that pass).  Whoever completes quad 0 has seen a line of every workgroup of
+// the group: all of them have read the launch count by then, and it moves on.
 __device__ inline int merge_quads(const MergeGeom &mg, int q_begin, int q_end, int wi, int nw, int lane,
                                   unsigned long long t0, unsigned long long limit) {
+    // s in the upper bits of the lane index, where reductions are cheap
     const int SL = 1 << mg.sl_log, qw = 16 >> mg.sl_log;
-    const int piece = lane & 3, s = (lane >> 2) & (SL - 1), qslot = lane >> (2 + mg.sl_log);
+    const int piece = lane & 3, qslot = (lane >> 2) & (qw - 1), s = lane >> (6 - mg.sl_log);
     for (int q0 = q_begin + wi * qw; q0 < q_end; q0 += nw * qw) {
         const int q = q0 + qslot;
         const bool valid = q < q_end;
         const int qc = valid ? q : q_end - 1;
         const int hd = qc / QUADS, quad = qc - hd * QUADS;
-        const float *base = mg.part_g + ((hd * QUADS + quad) * 4 + piece) * 4;
-        float run_m = -INFINITY, acc_w = 0.f;
-        floatx4 acc_o = {0.f, 0.f, 0.f, 0.f};
+        const float *base = mg.part_g + ((int64_t)(hd * QUADS + quad) * mg.nsplit * 4 + piece) * 4;
+        Fold acc = {-INFINITY, 0.f, floatx4{0.f, 0.f, 0.f, 0.f}};
         for (int b0 = 0; b0 < mg.nsplit; b0 += 8 * SL) {
-            uintx4 r[8];
-            const float *p[8];
-            bool need[8];
-            unsigned long long stale[8];
-#pragma unroll
-            for (int it = 0; it < 8; it++) {
-                const int sp = b0 + it * SL + s;
-                r[it] = uintx4{0u, 0u, 0u, 0u};
-                need[it] = valid && sp < mg.nsplit;
-                p[it] = base + (int64_t)(sp < mg.nsplit ? sp : 0) * kDecodePartFloats;
-                stale[it] = __ballot(need[it]);
-            }
-            while (true) {
-                ld_lines8(p, r, stale);  // only what has not arrived yet is loaded again
-                unsigned long long any = 0ull;
-#pragma unroll
-                for (int it = 0; it < 8; it++) {
-                    stale[it] = __ballot(need[it] && r[it][0] != mg.stamp32);
-                    any |= stale[it];
-                }
-                if (any == 0ull) {
-                    break;
-                }
-                if (wall_clock64() - t0 > limit) {
-                    return 1;
-                }
-                __builtin_amdgcn_s_sleep(2);
-            }
-            // log-sum-exp of each line from the bytes in its four pieces, then the batch's max
-            float lse[8];
-            float bm = -INFINITY;
-#pragma unroll
-            for (int it = 0; it < 8; it++) {
-                int bits = (int)(r[it][3] >> 24) << (8 * piece);
-                bits |= __builtin_amdgcn_update_dpp(0, bits, 0xB1, 0xf, 0xf, true);  // quad_perm [1,0,3,2]
-                bits |= __builtin_amdgcn_update_dpp(0, bits, 0x4E, 0xf, 0xf, true);  // quad_perm [2,3,0,1]
-                lse[it] = need[it] ? __int_as_float(bits) : -INFINITY;
-                bm = fmaxf(bm, lse[it]);
-            }
-            bm = reduce_splits(bm, mg.sl_log, [](float a, float b) { return fmaxf(a, b); });
-            const float m_new = fmaxf(run_m, bm);
-            if (m_new != -INFINITY) {
-                const float sc = (run_m == -INFINITY) ? 0.f : __expf(run_m - m_new);
-                acc_w *= sc;
-                acc_o *= sc;
-#pragma unroll
-                for (int it = 0; it < 8; it++) {
-                    const float wgt = (lse[it] == -INFINITY) ? 0.f : __expf(lse[it] - m_new);
-                    const floatx4 v = unpack_piece(r[it]);
-                    acc_w += wgt;
-#pragma unroll
-                    for (int e = 0; e < 4; e++) {
-                        acc_o[e] = __builtin_fmaf(wgt, v[e], acc_o[e]);
-                    }
-                }
-                run_m = m_new;
+            if (poll_lines(base, b0 + s, SL, mg.nsplit, valid, mg.stamp32, piece, t0, limit, acc)) {
+                return 1;
             }
         }
-        auto add = [](float a, float b) { return a + b; };
-        acc_w = reduce_splits(acc_w, mg.sl_log, add);
-#pragma unroll
-        for (int e = 0; e < 4; e++) {
-            acc_o[e] = reduce_splits(acc_o[e], mg.sl_log, add);
-        }
+        reduce_fold(acc, mg.sl_log);
+        TS(11);
         if (valid && s == 0) {
             // (1 / sum to one ulp, then a product: the values were cut to 22 bits on their way here)
             *reinterpret_cast<floatx4 *>(mg.out_g + hd * D + quad * 16 + piece * 4) =
-                acc_o * __builtin_amdgcn_rcpf(acc_w);
+                acc.o * __builtin_amdgcn_rcpf(acc.w);
+        }
+        if (q0 == 0 && lane == 0) {
+            __hip_atomic_store(mg.gen_word, mg.gen_next, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     }
     return 0;
@@ -367,10 +508,17 @@ struct DecodeShared {
     float mrun[2][16];  // running max after a round
     float l[W][16];     // sums per score wave, at the final running max
     float pnew[16];     // probability of the new token
+    __attribute__((aligned(16))) __half knew[D];  // its key, roped, fp16
+    __attribute__((aligned(16))) __half q[16][QPAD];  // the group's queries, roped, scaled, fp16
+    int q_ready;        // score waves that have left their part of the queries
     int m_ready;        // score waves that have left their maxes, over all rounds
     int p_ready;        // score waves that have left their part of P, over all rounds
     int p_done;         // output waves that are through with P, over all rounds
     int stored;         // output waves whose line stores have been performed
+    // the four score waves on one quad of the output: what each leaves for the first of them
+    float red[W][4][8];  // per wave and piece: max, sum, O[4]
+    int red_ready;
+    int red_fail;
 };
 
 // A wave waits for waves of its own workgroup (all resident by construction) through a counter in LDS.
@@ -406,6 +554,78 @@ __device__ inline float sum_over_c(float x) {
     return __uint_as_float(b[0]) + __uint_as_float(b[1]);
 }
 
+// The long-context shape: one quad per workgroup and many splits.  All four score waves work on the
+// quad, 64 split lanes in all, and the first of them finishes it from what the others leave in LDS.
+__device__ inline int merge_quad4(const MergeGeom &mg, DecodeShared &sh, int q, int wv, int lane,
+                                  unsigned long long t0, unsigned long long limit, uint32_t *flags) {
+    const int piece = lane & 3, s = wv * 16 + (lane >> 2);
+    const int hd = q / QUADS, quad = q - hd * QUADS;
+    const float *base = mg.part_g + ((int64_t)(hd * QUADS + quad) * mg.nsplit * 4 + piece) * 4;
+    Fold acc = {-INFINITY, 0.f, floatx4{0.f, 0.f, 0.f, 0.f}};
+    int failed = 0;
+    for (int b0 = 0; b0 < mg.nsplit && !failed; b0 += 8 * 64) {
+        failed = poll_lines(base, b0 + s, 64, mg.nsplit, true, mg.stamp32, piece, t0, limit, acc);
+    }
+    reduce_fold(acc, 4);
+    TS(4);
+    if (lane < 4) {
+        float *dst = &sh.red[wv][piece][0];
+        dst[0] = acc.m;
+        dst[1] = acc.w;
+        *reinterpret_cast<floatx4 *>(dst + 4) = acc.o;
+        if (failed) {
+            sh.red_fail = 1;
+        }
+    }
+    lds_signal(&sh.red_ready, lane);
+    if (wv != 0) {
+        return failed;
+    }
+    lds_wait_ge(&sh.red_ready, W, flags);
+    failed |= __hip_atomic_load(&sh.red_fail, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    if (failed) {
+        return 1;
+    }
+    if (lane < 4) {
+        float m_all = acc.m;
+#pragma unroll
+        for (int ww = 1; ww < W; ww++) {
+            m_all = fmaxf(m_all, sh.red[ww][piece][0]);
+        }
+        float f = (acc.m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(acc.m - m_all);
+        float wsum = acc.w * f;
+        floatx4 osum = acc.o * f;
+#pragma unroll
+        for (int ww = 1; ww < W; ww++) {
+            const float mw = sh.red[ww][piece][0];
+            f = (mw == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(mw - m_all);
+            wsum = __builtin_fmaf(sh.red[ww][piece][1], f, wsum);
+            const floatx4 ow = *reinterpret_cast<const floatx4 *>(&sh.red[ww][piece][4]);
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                osum[e] = __builtin_fmaf(ow[e], f, osum[e]);
+            }
+        }
+        TS(11);
+        *reinterpret_cast<floatx4 *>(mg.out_g + hd * D + quad * 16 + piece * 4) = osum * __builtin_amdgcn_rcpf(wsum);
+    }
+    if (q == 0 && lane == 0) {
+        __hip_atomic_store(mg.gen_word, mg.gen_next, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    return 0;
+}
+
+// A slice that was left behind has been written after all: whoever takes the flag off takes it off the
+// count of lost slices as well (once, however many redo it).
+__device__ inline void slice_redone(unsigned long long *claim, unsigned long long stamp, unsigned int *lost, int lane) {
+    if (lane == 0) {
+        const unsigned long long old = __hip_atomic_exchange(claim, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (old == stamp) {
+            __hip_atomic_fetch_add(lost, 0xffffffffu, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+}
+
 struct Geom {
     int lane, w, j, c, g, split;
     int tb, te, rounds;
@@ -419,11 +639,8 @@ __device__ inline void score_wave(const DecodeArgs &a, DecodeShared &sh, const G
     const int lane = ge.lane, w = ge.w, j = ge.j, c = ge.c, g = ge.g;
     const int L = a.s.L, G = a.s.G;
     const __half *Kg = a.k_cache + (int64_t)g * L * D;
-    const bool owner = ge.owner_wg && w == 0;
+    const bool owner = ge.owner_wg && w == W - 1;
 
-    int nk = ge.te - ge.tb < W ? ge.te - ge.tb : W;
-    half8 kf[4][4];
-    load_k_tile(Kg, L, (ge.tb + (w < nk ? w : 0)) * TILE, lane, kf);
     int pos[2] = {a.pos0, a.pos1};
     if (TYPE != GLM_ATTN_ROPE_DISABLED) {
         if (!a.pos_from_args) {
@@ -433,31 +650,46 @@ __device__ inline void score_wave(const DecodeArgs &a, DecodeShared &sh, const G
         pos[0] = clamp_position(pos[0], a.rope.table_positions, a.flags);
         pos[1] = clamp_position(pos[1], a.rope.table_positions, a.flags);
     }
-    RowRegs qreg;
+    // loads of a wave return in order: the small rows first, so that the queries can be prepared while
+    // the K tile is on its way
+    QPart qpart;
+    const int q_hd = 4 * w + (lane >> 4), q_d0 = (lane & 15) * 8;
     {
-        const int hd = j < G ? j : G - 1;  // lanes beyond the group read a valid row and are zeroed below
-        issue_row_loads<TYPE>(a.qkv + a.lay.q_off + (int64_t)(g * G + hd) * a.lay.head_stride, c, pos, a.rope, qreg);
+        const int hd = q_hd < G ? q_hd : G - 1;  // rows beyond the group read a valid row and are zeroed below
+        issue_q_part<TYPE>(a.qkv + a.lay.q_off + (int64_t)(g * G + hd) * a.lay.head_stride, q_d0, pos, a.rope, qpart);
     }
-    RowRegs kreg;
+    QPart kpart;  // the new token's k: lane l (and l + 16, ...) takes dims (l & 15) * 8 ..
     if (owner) {
-        issue_row_loads<TYPE>(a.qkv + a.lay.k_off + (int64_t)g * a.lay.head_stride, c, pos, a.rope, kreg);
+        issue_q_part<TYPE>(a.qkv + a.lay.k_off + (int64_t)g * a.lay.head_stride, q_d0, pos, a.rope, kpart);
     }
+    int nk = ge.te - ge.tb < W ? ge.te - ge.tb : W;
+    half8 kf[4][4];
+    load_k_tile(Kg, L, (ge.tb + (w < nk ? w : 0)) * TILE, lane, kf);
     TS(0);
+    *reinterpret_cast<half8 *>(&sh.q[q_hd][q_d0]) = finish_q_part<TYPE>(qpart, q_d0, a.scale, q_hd >= G);
+    lds_signal(&sh.q_ready, lane);
+    lds_wait_ge(&sh.q_ready, W, a.flags);
     half8 qf[4];
-    finish_row<TYPE>(qreg, a.scale, j >= G, qf);
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+        qf[t] = *reinterpret_cast<const half8 *>(&sh.q[j][t * 32 + c * 8]);
+    }
     float s_new = -INFINITY;  // score of the new token, in the wave that attends to it
     if (owner) {
         // chatglm.cpp:668-671: k (roped) of the new token goes to the cache as fp16
-        half8 kn[4];
-        finish_row<TYPE>(kreg, 1.0f, false, kn);
+        const half8 k8 = finish_q_part<TYPE>(kpart, q_d0, 1.0f, false);
+        if (lane < 16) {
+            *reinterpret_cast<half8 *>(a.k_cache + ((int64_t)g * L + a.p0) * D + q_d0) = k8;
+            *reinterpret_cast<half8 *>(&sh.knew[q_d0]) = k8;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
         const half8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
         floatx4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int t = 0; t < 4; t++) {
-            if (j == 0) {
-                *reinterpret_cast<half8 *>(a.k_cache + ((int64_t)g * L + a.p0) * D + t * 32 + c * 8) = kn[t];
-            }
-            acc = mfma16(j == 0 ? kn[t] : zero, qf[t], acc);  // row 0 of the product: the new key
+            const half8 kn = *reinterpret_cast<const half8 *>(&sh.knew[t * 32 + c * 8]);
+            acc = mfma16(j == 0 ? kn : zero, qf[t], acc);  // row 0 of the product: the new key
         }
         s_new = __shfl(acc[0], j);
     }
@@ -543,9 +775,9 @@ __device__ inline void score_wave(const DecodeArgs &a, DecodeShared &sh, const G
             sh.l[w][j] = l_run;
             if (w == 0) {
                 sh.mrun[r & 1][j] = m_new;
-                if (r == 0) {
-                    sh.pnew[j] = pn;
-                }
+            }
+            if (r == 0 && owner) {
+                sh.pnew[j] = pn;
             }
         }
         lds_signal(&sh.p_ready, lane);
@@ -600,19 +832,22 @@ __device__ inline void output_wave(const DecodeArgs &a, DecodeShared &sh, const 
         const float alpha = (m_run == -INFINITY) ? 0.f : __expf(m_run - m_new);
         m_run = m_new;
         if ((rt0 + nk) * TILE > a.p0) {
-            // V columns of keys that do not exist may hold anything (never written, or stale): zero them
+            // V columns of keys that do not exist may hold anything (never written, or stale): zero them.
+            // They can only be in the round's last tile.
 #pragma unroll
             for (int ks = 0; ks < 8; ks++) {
-                const int nv = a.p0 - (rt0 * TILE + ks * 32 + c * 8);  // keys of this lane's eight that exist
-                if (nv < 8) {
+                if (ks >= 2 * nk - 2 && ks < 2 * nk) {
+                    const int nv = a.p0 - (rt0 * TILE + ks * 32 + c * 8);  // keys of this lane's eight that exist
+                    uintx4 keep;
+#pragma unroll
+                    for (int dw = 0; dw < 4; dw++) {
+                        keep[dw] = nv >= 2 * dw + 2 ? 0xffffffffu : nv == 2 * dw + 1 ? 0x0000ffffu : 0u;
+                    }
 #pragma unroll
                     for (int jb = 0; jb < 2; jb++) {
-#pragma unroll
-                        for (int e = 0; e < 8; e++) {
-                            if (e >= nv) {
-                                vf[jb][ks][e] = (_Float16)0.f;
-                            }
-                        }
+                        uintx4 bits = __builtin_bit_cast(uintx4, vf[jb][ks]);
+                        bits &= keep;
+                        vf[jb][ks] = __builtin_bit_cast(half8, bits);
                     }
                 }
             }
@@ -696,6 +931,8 @@ __device__ inline void decode_body(const DecodeArgs &a, DecodeShared &sh) {
     mg.stamp32 = stamp32;
     mg.part_g = a.part + (int64_t)g * a.nsplit * kDecodePartFloats;
     mg.out_g = a.out + (int64_t)g * G * D;
+    mg.gen_word = &a.sync[g].gen;
+    mg.gen_next = decode_next_gen(gen);
     DecodeGroupSync *sy = a.sync + g;
     unsigned long long *claim = a.claim + (int64_t)g * kDecodeMaxSplits;
     const unsigned long long stamp = gen + 1ull;
@@ -705,18 +942,22 @@ __device__ inline void decode_body(const DecodeArgs &a, DecodeShared &sh) {
         if (a.nsplit == 1) {
             return;
         }
+#ifdef EXP_NO_MERGE
+        return;
+#endif
         // ---- grid-wide merge.  The score waves of every workgroup fold the quads of one slice of the
         // group's output from the lines of all splits, which they load past the caches and poll until
         // they carry this launch's stamp.  The poll is bounded: a wave whose wait runs out flags the
-        // slice as left behind, looks once more and goes on to exit.  An output wave takes a ticket
-        // once the lines of the whole workgroup have been performed; the holder of the last ticket
-        // knows that every partial is complete, merges the slices it finds flagged, zeroes the ticket
-        // counter for the next launch and bumps the launch count.  Two waves may merge the same slice;
-        // they then write identical values.
+        // slice as left behind, looks once more and goes on to exit.  Every workgroup looks for such
+        // flags once its own lines have been performed, and redoes the slices it finds flagged: the
+        // workgroup whose lines are performed last finds every partial complete and every flag that
+        // was raised before its look; a flag raised after that look is followed by a look that finds
+        // every partial complete.  Two waves may merge the same slice; they then write identical values.
         const int q_begin = split * qps;
         const int q_end = (split + 1) * qps < total_quads ? (split + 1) * qps : total_quads;
         const int qw = 16 >> mg.sl_log;
-        if (q_begin + w * qw >= q_end) {
+        const bool four = qps == 1 && a.nsplit > 64;  // all four waves on the one quad
+        if (q_begin >= q_end || (!four && q_begin + w * qw >= q_end)) {
             return;
         }
         const unsigned long long t0 = wall_clock64();
@@ -732,19 +973,24 @@ __device__ inline void decode_body(const DecodeArgs &a, DecodeShared &sh) {
             }
         }
         TS(6);
-        int failed = merge_quads(mg, q_begin, q_end, w, W, lane, t0, limit);
+        int failed = four ? merge_quad4(mg, sh, q_begin, w, lane, t0, limit, a.flags)
+                          : merge_quads(mg, q_begin, q_end, w, W, lane, t0, limit);
         TS(7);
-        if (failed) {
-            // Flag the slice for the holder of the last ticket (the slice's word, then a count in the
-            // ticket word, which that workgroup sees in the answer to its own ticket), then look once
-            // more: if that workgroup already has its ticket, every partial is complete by now and
-            // this attempt succeeds.  (The attempt starts after both are known to be in place.)
+        if (failed && (!four || w == 0)) {
+            // Flag the slice (its own word, then the group's), then look once more, on its own and at
+            // the whole slice.  (The look starts after the flags are known to be in place.)
             if (lane == 0) {
-                (void)__hip_atomic_exchange(claim + split, stamp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                (void)__hip_atomic_fetch_add(&sy->ticket, 0x10000u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                const unsigned long long old =
+                    __hip_atomic_exchange(claim + split, stamp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if (old != stamp) {
+                    __hip_atomic_fetch_add(&sy->lost, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+                __hip_atomic_store(&sy->flagged, stamp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
             wait_vm();
-            (void)merge_quads(mg, q_begin, q_end, w, W, lane, wall_clock64(), 0ull);
+            if (!merge_quads(mg, q_begin, q_end, 0, 1, lane, wall_clock64(), 0ull)) {
+                slice_redone(claim + split, stamp, &sy->lost, lane);
+            }
         }
         return;
     }
@@ -767,61 +1013,51 @@ __device__ inline void decode_body(const DecodeArgs &a, DecodeShared &sh) {
         }
         return;
     }
-    // ---- the workgroup's partial as stamped lines: O / sum and max + ln(sum) per head.  Lane (j, c)
+    // ---- the workgroup's partial as stamped lines: O / sum and the log-sum-exp per head.  Lane (j, c)
     // of output wave w holds piece c of quads 2 w and 2 w + 1 of head j.
     if (j < G) {
-        float *pw = a.part + ((int64_t)g * a.nsplit + split) * kDecodePartFloats;
+        float *pw = a.part + (int64_t)g * a.nsplit * kDecodePartFloats + split * 16;
         const float inv = l_tot > 0.f ? __builtin_amdgcn_rcpf(l_tot) : 0.f;
-        const unsigned int lse = __float_as_uint(l_tot > 0.f ? m_fin + __logf(l_tot) : -INFINITY);
+        const unsigned int lse =  // base 2: what the exponential instruction takes
+            __float_as_uint(l_tot > 0.f ? __builtin_fmaf(m_fin, 1.44269504088896340736f, __log2f(l_tot)) : -INFINITY);
 #pragma unroll
         for (int jb = 0; jb < 2; jb++) {
-            st_dev4(pw + ((j * QUADS + w * 2 + jb) * 4 + c) * 4, pack_piece(stamp32, o[jb] * inv, lse, c));
+            st_dev4(pw + (int64_t)(j * QUADS + w * 2 + jb) * a.nsplit * 16 + c * 4,
+                    pack_piece(stamp32, o[jb] * inv, lse, c));
         }
     }
     TS(5);
-    // ---- ticket, and the sweep if this workgroup holds the last one
+#ifdef EXP_NO_TICKET
+    return;
+#endif
+    // ---- once the lines of the whole workgroup have been performed: has anybody left a slice behind?
     wait_vm();  // this wave's line stores have been performed
     lds_signal(&sh.stored, lane);
     if (w != 0) {
         return;
     }
     lds_wait_ge(&sh.stored, W, a.flags);
-    unsigned int ticket = 0;
-    if (lane == 0) {
-        ticket = __hip_atomic_fetch_add(&sy->ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    ticket = __shfl(ticket, 0);
-    if ((ticket & 0xffffu) != (unsigned int)a.nsplit - 1u) {
-        return;
+    if (__hip_atomic_load(&sy->flagged, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != stamp) {
+        return;  // normally
     }
     TS(8);
-    // slices whose owners left before this ticket: normally none, and then nothing is scanned
-    if (ticket >> 16) {
-        const unsigned long long sweep_limit = a.spin_ticks > 10000 ? (unsigned long long)a.spin_ticks : 10000ull;
-        const int n_slices = (total_quads + qps - 1) / qps;
-        int lost = 0;
-        for (int sl0 = 0; sl0 < n_slices; sl0 += 64) {
-            unsigned long long cl = 0;
-            if (sl0 + lane < n_slices) {
-                cl = __hip_atomic_load(claim + sl0 + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            }
-            unsigned long long left = __ballot(sl0 + lane < n_slices && cl == stamp);
-            while (left) {
-                const int sl = sl0 + __builtin_ctzll(left);
-                left &= left - 1;
-                const int qb = sl * qps;
-                const int qe = (sl + 1) * qps < total_quads ? (sl + 1) * qps : total_quads;
-                lost |= merge_quads(mg, qb, qe, 0, 1, lane, wall_clock64(), sweep_limit);
+    const unsigned long long sweep_limit = a.spin_ticks > 10000 ? (unsigned long long)a.spin_ticks : 10000ull;
+    const int n_slices = (total_quads + qps - 1) / qps;
+    for (int sl0 = 0; sl0 < n_slices; sl0 += 64) {
+        unsigned long long cl = 0;
+        if (sl0 + lane < n_slices) {
+            cl = __hip_atomic_load(claim + sl0 + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        unsigned long long left = __ballot(sl0 + lane < n_slices && cl == stamp);
+        while (left) {
+            const int sl = sl0 + __builtin_ctzll(left);
+            left &= left - 1;
+            const int qb = sl * qps;
+            const int qe = (sl + 1) * qps < total_quads ? (sl + 1) * qps : total_quads;
+            if (!merge_quads(mg, qb, qe, 0, 1, lane, wall_clock64(), sweep_limit)) {
+                slice_redone(claim + sl, stamp, &sy->lost, lane);
             }
         }
-        if (lost && lane == 0) {
-            atomicOr(a.flags, kFlagMergeIncomplete);
-        }
-    }
-    // the launch is over for this group: words for the next one
-    if (lane == 0) {
-        __hip_atomic_store(&sy->ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(&sy->gen, decode_next_gen(gen), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     TS(9);
 }
@@ -829,10 +1065,13 @@ __device__ inline void decode_body(const DecodeArgs &a, DecodeShared &sh) {
 __global__ __launch_bounds__(kBlock) void decode_kernel(DecodeArgs a) {
     __shared__ DecodeShared sh;
     if (threadIdx.x == 0) {
+        sh.q_ready = 0;
         sh.m_ready = 0;
         sh.p_ready = 0;
         sh.p_done = 0;
         sh.stored = 0;
+        sh.red_ready = 0;
+        sh.red_fail = 0;
     }
     __syncthreads();
     switch (a.rope.pairs > 0 ? a.rope.type : GLM_ATTN_ROPE_DISABLED) {

@@ -544,6 +544,12 @@ int glm_attn_device_flags(glm_attn_ctx *ctx, uint32_t *flags) {
     DeviceGuard guard(ctx->desc.device);
     HIP_TRY(ctx, hipDeviceSynchronize());
     HIP_TRY(ctx, hipMemcpy(flags, ctx->flags, sizeof(uint32_t), hipMemcpyDeviceToHost));
+    // slices of a decode output that their owners left behind and nobody redid
+    std::vector<DecodeGroupSync> sync((size_t)ctx->shape.kvh);
+    HIP_TRY(ctx, hipMemcpy(sync.data(), ctx->sync, sync.size() * sizeof(DecodeGroupSync), hipMemcpyDeviceToHost));
+    for (const DecodeGroupSync &g : sync) {
+        if (g.lost != 0) *flags |= kFlagMergeIncomplete;
+    }
     return GLM_ATTN_OK;
 }
 

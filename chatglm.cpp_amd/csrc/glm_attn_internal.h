@@ -22,20 +22,19 @@ constexpr int kDecodeMaxWaves = 4;   // tile waves per workgroup of the decode k
 constexpr int kDecodeMaxSplits = 512;  // workgroups per KV group of the decode kernel
 // floats of one (group, split) partial of the decode kernel: 16 heads x 8 lines of 64 bytes
 constexpr int kDecodePartFloats = 16 * 8 * 16;
-constexpr int kDecodeHintShards = 4;   // arrival counters per KV group, one 64-byte line each
 constexpr int kTimelineSlots = 4096;   // waves recorded by the instrumented build of the decode kernel
 constexpr uint32_t kFlagPositionClamped = 1u;
 constexpr uint32_t kFlagMergeIncomplete = 2u;  // a slice of a decode output was left unwritten
 
-// Hand-over words of the decode kernel, one set per KV group.
+// Hand-over words of the decode kernel, one set per KV group (a 64-byte line of its own each).
 struct DecodeGroupSync {
-    unsigned long long gen;   // launches of this group completed so far (with more than one split)
-    unsigned int hint_base;   // sum of the hint counters when the current launch began
-    unsigned int ticket;      // low 16 bits: workgroups whose lines are performed; above: slices left behind
-    unsigned int pad[12];
-    unsigned int hint[kDecodeHintShards][16];  // workgroups that have issued their lines, ever (word 0 of each line)
+    unsigned long long gen;      // launches of this group completed so far (with more than one split)
+    unsigned long long flagged;  // launch (gen + 1) in which a slice was last left behind by its owner
+    unsigned int lost;           // slices left behind and not (yet) redone by anybody, over all launches
+    unsigned int pad0;
+    unsigned long long pad[5];
 };
-static_assert(sizeof(DecodeGroupSync) == 64 * (1 + kDecodeHintShards), "one line per counter");
+static_assert(sizeof(DecodeGroupSync) == 64, "one line per group");
 
 // The 32-bit stamp of the lines written by the launch that follows `gen` completed ones.  It is never
 // 0 (what a zero-filled exchange buffer holds): decode_next_gen skips the count whose stamp would be.
