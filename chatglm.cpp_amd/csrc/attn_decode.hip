@@ -346,39 +346,66 @@ __device__ inline float reduce_splits(float x, int sl_log, F op) {
     return x;
 }
 
-// One round of a poll: the lines that have shown up since the last round are folded into the lane's
-// running (max, sum, O), so that what is left to do after the last line has arrived is that line and the
-// reduction over the lanes.  A line counts when all four of its pieces carry the stamp (its log-sum-exp
-// is spread over them).  `want` has a bit per line this lane still needs; returns the lanes' union.
+// Polls lines `first + it * step` (it = 0 .. 7, those below nsplit) of one (quad, piece) until all have
+// arrived, then folds them into the lane's (max, sum, O) in the order of their index: the result does not
+// depend on the order in which the lines showed up.  A line counts when all four of its pieces carry the
+// stamp (its log-sum-exp is spread over them).  Returns 1 when the wait ran out.
 struct Fold {
     float m, w;
     floatx4 o;
 };
-__device__ inline unsigned long long fold_round(const uintx4 (&r)[8], unsigned int &want, unsigned int stamp32,
-                                                int piece, unsigned long long (&pending)[8], Fold &acc) {
-    // which lines are new, and the base-2 log-sum-exp of each from the bytes in its four pieces
-    float lse[8];
-    float m_new = acc.m;
-    unsigned int got = 0;
+__device__ inline int poll_lines(const float *base, int first, int step, int nsplit, bool valid, unsigned int stamp32,
+                                 int piece, unsigned long long t0, unsigned long long limit, Fold &acc) {
+    uintx4 r[8];
+    const float *p[8];
+    bool need[8];
+    unsigned long long pending[8];
 #pragma unroll
     for (int it = 0; it < 8; it++) {
-        lse[it] = -INFINITY;
-        if (pending[it] == 0ull) {
-            continue;
+        const int sp = first + it * step;
+        r[it] = uintx4{0u, 0u, 0u, 0u};
+        need[it] = valid && sp < nsplit;
+        p[it] = base + (sp < nsplit ? sp : 0) * 16;
+        pending[it] = __ballot(need[it]);
+    }
+    TS(13);
+    while (true) {
+        const unsigned long long now = wall_clock64();  // read while the loads are on their way
+        ld_lines8(p, r, pending);                       // only what has not arrived yet is loaded again
+        TSCOUNT(14);
+        TS(15);
+        unsigned long long any = 0ull;
+#pragma unroll
+        for (int it = 0; it < 8; it++) {
+            if (pending[it] != 0ull) {
+                // all four pieces of a line: and over the quad of lanes
+                int ok = !need[it] || r[it][0] == stamp32;
+                ok &= __builtin_amdgcn_update_dpp(0, ok, 0xB1, 0xf, 0xf, true);  // quad_perm [1,0,3,2]
+                ok &= __builtin_amdgcn_update_dpp(0, ok, 0x4E, 0xf, 0xf, true);  // quad_perm [2,3,0,1]
+                pending[it] = __ballot(!ok);
+                any |= pending[it];
+            }
         }
-        int ok = ((want >> it) & 1u) && r[it][0] == stamp32;
-        ok &= __builtin_amdgcn_update_dpp(0, ok, 0xB1, 0xf, 0xf, true);  // quad_perm [1,0,3,2]
-        ok &= __builtin_amdgcn_update_dpp(0, ok, 0x4E, 0xf, 0xf, true);  // quad_perm [2,3,0,1]
+        if (any == 0ull) {
+            break;
+        }
+        if (now - t0 > limit) {
+            return 1;
+        }
+        __builtin_amdgcn_s_sleep(1);
+    }
+    TS(12);
+    // the base-2 log-sum-exp of each line from the bytes in its four pieces, and the new max
+    float lse[8];
+    float m_new = acc.m;
+#pragma unroll
+    for (int it = 0; it < 8; it++) {
         int bits = (int)(r[it][3] >> 24) << (8 * piece);
         bits |= __builtin_amdgcn_update_dpp(0, bits, 0xB1, 0xf, 0xf, true);
         bits |= __builtin_amdgcn_update_dpp(0, bits, 0x4E, 0xf, 0xf, true);
-        if (ok) {
-            got |= 1u << it;
-            lse[it] = __int_as_float(bits);
-            m_new = fmaxf(m_new, lse[it]);
-        }
+        lse[it] = need[it] ? __int_as_float(bits) : -INFINITY;
+        m_new = fmaxf(m_new, lse[it]);
     }
-    want &= ~got;
     if (m_new != -INFINITY) {
         const float sc = __builtin_amdgcn_exp2f(acc.m - m_new);  // exp2(-inf) = 0 for the first lines
         acc.w *= sc;
@@ -386,10 +413,7 @@ __device__ inline unsigned long long fold_round(const uintx4 (&r)[8], unsigned i
         acc.m = m_new;
 #pragma unroll
         for (int it = 0; it < 8; it++) {
-            if (pending[it] == 0ull) {
-                continue;
-            }
-            const float wgt = __builtin_amdgcn_exp2f(lse[it] - m_new);  // 0 for lines that are not new
+            const float wgt = __builtin_amdgcn_exp2f(lse[it] - m_new);  // 0 for lines that are not there
             const floatx4 v = unpack_piece(r[it]);
             acc.w += wgt;
 #pragma unroll
@@ -398,50 +422,7 @@ __device__ inline unsigned long long fold_round(const uintx4 (&r)[8], unsigned i
             }
         }
     }
-    unsigned long long any = 0ull;
-#pragma unroll
-    for (int it = 0; it < 8; it++) {
-        if (pending[it] != 0ull) {
-            pending[it] = __ballot((want >> it) & 1u);
-            any |= pending[it];
-        }
-    }
-    return any;
-}
-
-// Polls and folds lines `first + it * step` (it = 0 .. 7, those below nsplit) of one (quad, piece) until
-// all have arrived.  Returns 1 when the wait ran out.
-__device__ inline int poll_lines(const float *base, int first, int step, int nsplit, bool valid, unsigned int stamp32,
-                                 int piece, unsigned long long t0, unsigned long long limit, Fold &acc) {
-    uintx4 r[8];
-    const float *p[8];
-    unsigned int want = 0;  // bit it: this lane still needs line it
-    unsigned long long pending[8];
-#pragma unroll
-    for (int it = 0; it < 8; it++) {
-        const int sp = first + it * step;
-        r[it] = uintx4{0u, 0u, 0u, 0u};
-        const bool need = valid && sp < nsplit;
-        want |= need ? 1u << it : 0u;
-        p[it] = base + (sp < nsplit ? sp : 0) * 16;
-        pending[it] = __ballot(need);
-    }
-    TS(13);
-    while (true) {
-        const unsigned long long now = wall_clock64();  // read while the loads are on their way
-        ld_lines8(p, r, pending);                       // only what has not arrived yet is loaded again
-        TSCOUNT(14);
-        TS(15);
-        const unsigned long long any = fold_round(r, want, stamp32, piece, pending, acc);
-        TS(12);
-        if (any == 0ull) {
-            return 0;
-        }
-        if (now - t0 > limit) {
-            return 1;
-        }
-        __builtin_amdgcn_s_sleep(1);
-    }
+    return 0;
 }
 
 // What ends a slice: the (max, sum, O) of all lanes of a piece merged, normalised and stored.
