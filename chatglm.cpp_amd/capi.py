@@ -11,7 +11,7 @@ _PKG = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_PKG, "libglm_attn.so")
 CSRC = os.path.join(_PKG, "csrc")
 
-OK, EINVAL, ERANGE, ENOMEM, EHIP, EUNSUPPORTED = 0, -1, -2, -3, -4, -5
+OK, EINVAL, ERANGE, ENOMEM, EHIP, EUNSUPPORTED, ESTATIC = 0, -1, -2, -3, -4, -5, -6
 ROPE_GPTJ, ROPE_NEOX, ROPE_CHATGLM, ROPE_CHATGLM2, ROPE_DISABLED = 0, 2, 4, 8, 10000
 MASK_CAUSAL, MASK_CHATGLM = 0, 1
 MASK_RULE_REFERENCE, MASK_RULE_CAUSAL_OFFSET = 0, 1
@@ -19,7 +19,7 @@ MASK_RULE_REFERENCE, MASK_RULE_CAUSAL_OFFSET = 0, 1
 # every symbol include/glm_attn.h declares
 SYMBOLS = [
     "glm_attn_default_desc", "glm_attn_kv_bytes", "glm_attn_create", "glm_attn_destroy", "glm_attn_cache_ptrs",
-    "glm_attn_forward", "glm_attn_rope_append", "glm_attn_decode", "glm_attn_prefill",
+    "glm_attn_forward", "glm_attn_rope_append", "glm_attn_decode", "glm_attn_decode_static", "glm_attn_prefill",
     "glm_attn_load_prefix_cache", "glm_attn_position_ids_glm2", "glm_attn_position_ids_glm",
     "glm_attn_attention_mask_glm", "glm_attn_scale_add", "glm_attn_device_flags", "glm_attn_set_spin_limit_us", "glm_attn_last_hip_error", "glm_attn_strerror",
     "glm_attn_version",
@@ -164,6 +164,8 @@ def lib():
     L.glm_attn_rope_append.restype = c.c_int
     L.glm_attn_decode.argtypes = [P, c.c_int32, P, P, P, c.c_int32, P, P]
     L.glm_attn_decode.restype = c.c_int
+    L.glm_attn_decode_static.argtypes = [P, c.c_int32, P, P, P, c.c_int32, P, P]
+    L.glm_attn_decode_static.restype = c.c_int
     L.glm_attn_prefill.argtypes = [P, c.c_int32, P, c.c_int64, P, P, c.c_int32, c.c_int32, P, P]
     L.glm_attn_prefill.restype = c.c_int
     L.glm_attn_load_prefix_cache.argtypes = [P, c.c_int32, P, P]
@@ -240,6 +242,10 @@ class GlmAttnError(RuntimeError):
         super().__init__(f"{what}: {lib().glm_attn_strerror(status).decode()} (status {status})")
 
 
+def strerror(status):
+    return lib().glm_attn_strerror(status).decode()
+
+
 def check(status, what):
     if status != OK:
         raise GlmAttnError(status, what)
@@ -304,6 +310,15 @@ class Context:
         return lib().glm_attn_decode(self.handle, layer, qkv_ptr, position_ids_ptr,
                                      ctypes.cast(hp, ctypes.c_void_p) if hp is not None else None, n_past, out_ptr,
                                      stream)
+
+    def decode_static(self, layer, qkv_ptr, n_past, out_ptr, position_ids_ptr=None, position_ids_host=None,
+                      stream=None):
+        hp = None
+        if position_ids_host is not None:
+            hp = (ctypes.c_int32 * len(position_ids_host))(*[int(x) for x in position_ids_host])
+        return lib().glm_attn_decode_static(self.handle, layer, qkv_ptr, position_ids_ptr,
+                                            ctypes.cast(hp, ctypes.c_void_p) if hp is not None else None, n_past,
+                                            out_ptr, stream)
 
     def prefill(self, layer, qkv_ptr, position_ids_ptr, qlen, n_past, out_ptr, attention_mask_ptr=None,
                 qkv_row_stride=0, stream=None):

@@ -898,7 +898,7 @@ __device__ inline void decode_body(const DecodeArgs &a, DecodeShared &sh) {
     // The launch count stamps this launch's lines.  Every lane reads it (no branch, one request per
     // wave) among its first loads: no workgroup can have finished before that.
     const unsigned long long gen = __hip_atomic_load(&a.sync[g].gen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    const unsigned int stamp32 = decode_stamp(gen);
+    const unsigned int stamp32 = a.stamp_groups ? decode_stamp_grouped(gen, g) : decode_stamp(gen);
 
     const int total_quads = G * QUADS;
     const int qps = (total_quads + a.nsplit - 1) / a.nsplit;  // quads per slice

@@ -41,6 +41,43 @@ struct glm_attn_ctx {
 
 namespace {
 
+// ---- exchange memory of glm_attn_decode_static: the split partials and hand-over words of one decode
+// launch, for callers that must not allocate.  One copy per device, there from the moment the library is
+// loaded until the process ends; every call on a device uses that device's copy.
+constexpr int kStaticMaxGroups = 32;  // KV groups
+constexpr int kStaticMaxParts = 256;  // (group, split) partials of one launch = workgroups of the launch
+struct StaticScratch {
+    DecodeGroupSync sync[kStaticMaxGroups];
+    unsigned long long claim[kStaticMaxGroups][kDecodeMaxSplits];
+    float part[(size_t)kStaticMaxParts * kDecodePartFloats];
+};
+constexpr int kMaxDevices = 64;
+
+}  // namespace
+
+// 2.2 MB.  In host code this name is a stand-in for the symbol, not a device address: the address on a
+// device comes from hipGetSymbolAddress (scratch_on_device below), and only that is handed to kernels.
+static __device__ __align__(256) unsigned char scratch[sizeof(StaticScratch)];
+
+namespace {
+
+StaticScratch *g_scratch_ptr[kMaxDevices];  // per device, null until asked for
+
+// The address of `scratch` on the current device (which must be `device`).
+hipError_t scratch_on_device(int device, StaticScratch **out) {
+    *out = nullptr;
+    if (device < 0 || device >= kMaxDevices) return hipErrorInvalidDevice;
+    if (!g_scratch_ptr[device]) {
+        void *p = nullptr;
+        hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return e;
+        if (!p) return hipErrorInvalidSymbol;
+        g_scratch_ptr[device] = static_cast<StaticScratch *>(p);
+    }
+    *out = g_scratch_ptr[device];
+    return hipSuccess;
+}
+
 #define HIP_TRY(ctx, expr)                         \
     do {                                           \
         hipError_t e_ = (expr);                    \
@@ -213,8 +250,10 @@ AttendArgs make_attend(glm_attn_ctx *c, int layer, int qlen, int n_past, int cau
     return aa;
 }
 
+// `shared`: null, or the device's static exchange memory to use in place of the context's own
 int do_decode(glm_attn_ctx *c, int layer, const float *qkv, const int32_t *position_ids,
-              const int32_t *position_ids_host, int n_past, float *out, hipStream_t stream) {
+              const int32_t *position_ids_host, int n_past, float *out, hipStream_t stream,
+              StaticScratch *shared = nullptr) {
     DecodeArgs da;
     da.qkv = qkv;
     da.lay = call_layout(c, 0);
@@ -244,15 +283,17 @@ int do_decode(glm_attn_ctx *c, int layer, const float *qkv, const int32_t *posit
     int nsplit = n_tiles < 1 ? 1 : n_tiles;
     if (nsplit > cu_share) nsplit = cu_share;
     if (nsplit > c->max_splits) nsplit = c->max_splits;
+    if (shared && nsplit > kStaticMaxParts / c->shape.kvh) nsplit = kStaticMaxParts / c->shape.kvh;
     da.nsplit = nsplit;
     da.tiles_q = n_tiles / nsplit;
     da.tiles_r = n_tiles % nsplit;
-    da.part = c->part;
+    da.part = shared ? shared->part : c->part;
     da.out = out;
     da.flags = c->flags;
-    da.sync = c->sync;
-    da.claim = c->claim;
+    da.sync = shared ? shared->sync : c->sync;
+    da.claim = shared ? &shared->claim[0][0] : c->claim;
     da.spin_ticks = c->spin_ticks;
+    da.stamp_groups = shared ? 1 : 0;
     HIP_TRY(c, launch_decode(da, stream));
     return GLM_ATTN_OK;
 }
@@ -338,6 +379,14 @@ int glm_attn_create(const glm_attn_desc *desc, glm_attn_ctx **out_ctx) {
         return GLM_ATTN_EHIP;
     }
     c->num_cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+    {
+        // set-up is where the address of the static exchange memory on this device is looked up
+        StaticScratch *unused;
+        if (scratch_on_device(desc->device, &unused) != hipSuccess) {
+            delete c;
+            return GLM_ATTN_EHIP;
+        }
+    }
 
 #define CREATE_TRY(expr)                               \
     do {                                               \
@@ -453,6 +502,19 @@ int glm_attn_decode(glm_attn_ctx *ctx, int32_t layer, const float *qkv, const in
     if (!ctx->fast || !aligned16(qkv)) return GLM_ATTN_EUNSUPPORTED;
     DeviceGuard guard(ctx->desc.device);
     return do_decode(ctx, layer, qkv, position_ids, position_ids_host, n_past, out, (hipStream_t)stream);
+}
+
+int glm_attn_decode_static(glm_attn_ctx *ctx, int32_t layer, const float *qkv, const int32_t *position_ids,
+                           const int32_t *position_ids_host, int32_t n_past, float *out, void *stream) {
+    int rc = check_call(ctx, layer, 1, n_past);
+    if (rc != GLM_ATTN_OK) return rc;
+    if (!qkv || !out) return GLM_ATTN_EINVAL;
+    if (!ctx->fast || !aligned16(qkv)) return GLM_ATTN_EUNSUPPORTED;
+    if (ctx->shape.kvh > kStaticMaxGroups) return GLM_ATTN_ESTATIC;
+    DeviceGuard guard(ctx->desc.device);
+    StaticScratch *shared;
+    HIP_TRY(ctx, scratch_on_device(ctx->desc.device, &shared));  // looked up in glm_attn_create: no work here
+    return do_decode(ctx, layer, qkv, position_ids, position_ids_host, n_past, out, (hipStream_t)stream, shared);
 }
 
 int glm_attn_prefill(glm_attn_ctx *ctx, int32_t layer, const float *qkv, int64_t qkv_row_stride,
@@ -575,6 +637,8 @@ const char *glm_attn_strerror(int status) {
         return "HIP runtime error";
     case GLM_ATTN_EUNSUPPORTED:
         return "shape not supported by this entry point";
+    case GLM_ATTN_ESTATIC:
+        return "more KV groups than the static exchange memory of glm_attn_decode_static has room for (32)";
     default:
         return "unknown status";
     }

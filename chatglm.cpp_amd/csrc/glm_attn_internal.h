@@ -39,6 +39,12 @@ static_assert(sizeof(DecodeGroupSync) == 64, "one line per group");
 // The 32-bit stamp of the lines written by the launch that follows `gen` completed ones.  It is never
 // 0 (what a zero-filled exchange buffer holds): decode_next_gen skips the count whose stamp would be.
 __host__ __device__ inline unsigned int decode_stamp(unsigned long long gen) { return (unsigned int)(gen + 1ull); }
+// The same for exchange memory that contexts of different shapes share: the KV group is part of the stamp
+// (5 bits), so that a line can only be taken for one of the group that wrote it, whatever region of the
+// memory that group's lines occupied then; 27 bits of the launch count, never 0.
+__host__ __device__ inline unsigned int decode_stamp_grouped(unsigned long long gen, int group) {
+    return ((unsigned int)group << 27) | (unsigned int)(gen % 0x7ffffffull + 1ull);
+}
 __host__ __device__ inline unsigned long long decode_next_gen(unsigned long long gen) {
     const unsigned long long next = gen + 1ull;
     return decode_stamp(next) == 0u ? next + 1ull : next;
@@ -112,6 +118,7 @@ struct DecodeArgs {
     DecodeGroupSync *sync;      // [kvh]
     unsigned long long *claim;  // [kvh][kDecodeMaxSplits] launch (gen + 1) that last left each slice behind
     long long spin_ticks;       // bound on the wait for the other workgroups, in 100 MHz ticks
+    int stamp_groups;           // 1: stamps carry the KV group (exchange memory shared between contexts)
 };
 
 // activations of BasicMLP / BasicGLU (chatglm.cpp:444-454), shared by the elementwise kernel and the fused Linear

@@ -33,7 +33,8 @@ typedef enum glm_attn_status {
     GLM_ATTN_ERANGE = -2,       /* nvt + n_past + qlen > cache rows, layer out of range, qlen > max_qlen */
     GLM_ATTN_ENOMEM = -3,       /* device or host allocation failed */
     GLM_ATTN_EHIP = -4,         /* a HIP call failed; see glm_attn_last_hip_error */
-    GLM_ATTN_EUNSUPPORTED = -5  /* shape outside what the kernels are written for */
+    GLM_ATTN_EUNSUPPORTED = -5, /* shape outside what the kernels are written for */
+    GLM_ATTN_ESTATIC = -6       /* beyond the fixed size of glm_attn_decode_static's exchange memory */
 } glm_attn_status;
 
 /* Same numeric values as the reference's enum class RopeType (chatglm.h:93-99). */
@@ -133,6 +134,21 @@ int glm_attn_rope_append(glm_attn_ctx *ctx, int32_t layer, const float *qkv, int
    the split partials in one launch.  EUNSUPPORTED unless d == 128, h / kvh <= 16 and L % 8 == 0. */
 int glm_attn_decode(glm_attn_ctx *ctx, int32_t layer, const float *qkv, const int32_t *position_ids,
                     const int32_t *position_ids_host, int32_t n_past, float *out, void *stream);
+
+/* glm_attn_decode for callers that cannot allocate device memory and want no allocation of the library's
+   behind their call either (code under HIP graph capture, tight serving loops, harnesses that forbid
+   hipMalloc).  It has no counterpart in the reference.  Same arguments, same kernel and same result as
+   glm_attn_decode, but the split partials and the hand-over words of the launch live in a device array
+   that is part of the library's code object (2.2 MB on every GPU the library runs on, held until the
+   process ends) instead of in memory of the context; the call itself allocates and frees nothing.
+   Limit: at most 32 KV groups (GLM_ATTN_ESTATIC beyond), at most 256 workgroups per launch (the split
+   count is cut to fit).  All calls on one GPU share that GPU's array, whatever their context: calls that
+   overlap in time on one GPU (two streams, two threads) race and give wrong results; calls in stream
+   order on one stream at a time are fine, also from different contexts in turn.  Nothing needs to be
+   cleared between calls: what a launch reads of the array it has written itself, under a stamp that no
+   earlier launch used. */
+int glm_attn_decode_static(glm_attn_ctx *ctx, int32_t layer, const float *qkv, const int32_t *position_ids,
+                           const int32_t *position_ids_host, int32_t n_past, float *out, void *stream);
 
 /* forward through rope+append and the MFMA prefill kernel.  Same shape limits as decode. */
 int glm_attn_prefill(glm_attn_ctx *ctx, int32_t layer, const float *qkv, int64_t qkv_row_stride,

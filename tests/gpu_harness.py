@@ -155,6 +155,10 @@ class Pair:
             st = self.ctx.decode(layer, qkv_d.data_ptr(), n_past, out_d.data_ptr(),
                                  position_ids_ptr=None if host_pos else pos_d.data_ptr(),
                                  position_ids_host=pos if host_pos else None)
+        elif entry == "decode_static":
+            st = self.ctx.decode_static(layer, qkv_d.data_ptr(), n_past, out_d.data_ptr(),
+                                        position_ids_ptr=None if host_pos else pos_d.data_ptr(),
+                                        position_ids_host=pos if host_pos else None)
         elif entry == "prefill":
             st = self.ctx.prefill(layer, qkv_d.data_ptr(), pos_d.data_ptr(), qlen, n_past, out_d.data_ptr(),
                                   attention_mask_ptr=mp)
