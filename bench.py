@@ -60,6 +60,49 @@ def fill_cache_normal(torch, kv, seed):
         view[o:o + m] = torch.randn(m, generator=g, device=kv.device, dtype=torch.float32).to(torch.float16)
 
 
+def read_ceilings(torch, pkg, kv, layer_halfs, stream, warmup, steps):
+    """Kernels that only load, launched like the decode step: LAYERS launches back to back on one stream, each
+    over another layer's 32 MiB of cache, timed with events on that stream."""
+    lib = pkg.lib()
+    sink = torch.zeros(1, dtype=torch.float32, device=kv.device)
+    sh = stream.cuda_stream
+    layer_bytes = layer_halfs * 2
+    base = kv.data_ptr()
+
+    def run(pattern, per_launch_bytes, launches, whole=False):
+        def step():
+            for l in range(launches):
+                ptr = base if whole else base + l * layer_bytes
+                st = lib.glm_bench_read(pattern, ptr, MAX_LENGTH, KVH, per_launch_bytes, sink.data_ptr(), sh)
+                if st != 0:
+                    pkg.check(st, "glm_bench_read")
+
+        with torch.cuda.stream(stream):
+            for _ in range(warmup):
+                step()
+            torch.cuda.synchronize()
+            e0 = torch.cuda.Event(enable_timing=True)
+            e1 = torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            for _ in range(steps):
+                step()
+            e1.record(stream)
+            torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) * 1e3 / (steps * launches)
+        return {"us_per_launch": round(us, 3), "bytes_per_launch": per_launch_bytes,
+                "gbs": round(per_launch_bytes / (us * 1e-6) / 1e9, 1) if per_launch_bytes else None,
+                "frac_of_hbm_peak": round(per_launch_bytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)
+                if per_launch_bytes else None}
+
+    out = {"workload": f"{LAYERS} launches back to back per step, one layer's caches (32 MiB) per launch, "
+                       "256 workgroups of 8 waves, nothing but loads"}
+    out["empty_launch"] = run(pkg.BENCH_EMPTY, 0, LAYERS)
+    out["linear_read_per_launch"] = run(pkg.BENCH_READ_LINEAR, layer_bytes, LAYERS)
+    out["decode_pattern_read_per_launch"] = run(pkg.BENCH_READ_DECODE_PATTERN, layer_bytes, LAYERS)
+    out["one_long_streaming_launch"] = run(pkg.BENCH_READ_STREAM, layer_bytes * LAYERS, 1, whole=True)
+    return out
+
+
 class optional_section:
     """The sections beyond the contract's line (projections, whole layers, whole model) must not take the line with
     them: an exception inside one is recorded as that section's "error" and the run goes on."""
@@ -89,10 +132,20 @@ def main():
     ap.add_argument("--skip-linear", action="store_true", help="do not time the two projections around the path")
     ap.add_argument("--skip-layer", action="store_true", help="do not time whole decoder layers")
     ap.add_argument("--skip-model", action="store_true", help="do not time the whole model (C++ host classes)")
+    ap.add_argument("--ceiling", action="store_true",
+                    help="also time kernels that only read (one layer's caches per launch in address order and in "
+                         "the decode kernel's order, an empty launch, one long streaming launch): what this GPU "
+                         "gives a launch shaped like the decode kernel's")
+    ap.add_argument("--ceiling-only", action="store_true", help="time only those read kernels (for profiling)")
+    ap.add_argument("--decode-only", action="store_true", help="time only the decode step (for profiling)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB device copy (known size) so that FETCH_SIZE / WRITE_SIZE "
                          "counters of a profiled run can be scaled")
     args = ap.parse_args()
+    if args.ceiling_only:
+        args.ceiling = True
+    if args.decode_only or args.ceiling_only:
+        args.skip_cpu = args.skip_prefill = args.skip_linear = args.skip_layer = args.skip_model = True
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus must be 1 (no multi-GPU path exists)", file=sys.stderr)
         sys.exit(2)
@@ -129,8 +182,13 @@ def main():
     stream = torch.cuda.Stream()
     sh = stream.cuda_stream
 
+    # ------------------------------------------------------------------ read ceilings
+    if args.ceiling:
+        with optional_section(result, "ceiling"):
+            result["ceiling"] = read_ceilings(torch, pkg, kv, layer_halfs, stream, args.warmup, args.steps)
+
     # ------------------------------------------------------------------ decode
-    if not args.prefill_only:
+    if not args.prefill_only and not args.ceiling_only:
         qkv = torch.randn(LAYERS, width, generator=gen, device=dev, dtype=torch.float32)
         out = torch.zeros(LAYERS, H * D, device=dev, dtype=torch.float32)
         pos_host = [N_PAST_DECODE]

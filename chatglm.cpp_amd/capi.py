@@ -40,6 +40,8 @@ MODEL_FILE_SYMBOLS = [
     "glm_model_file_data", "glm_model_file_tensor_count", "glm_model_file_tensor", "glm_model_file_find",
     "glm_model_file_upload",
 ]
+BENCH_SYMBOLS = ["glm_bench_read"]
+BENCH_READ_LINEAR, BENCH_READ_DECODE_PATTERN, BENCH_READ_STREAM, BENCH_EMPTY = 0, 1, 2, 3
 MODEL_F32, MODEL_F16, MODEL_Q4_0, MODEL_Q4_1, MODEL_Q5_0, MODEL_Q5_1, MODEL_Q8_0 = 0, 1, 2, 3, 6, 7, 8
 
 
@@ -214,6 +216,8 @@ def lib():
     L.glm_block_gated_activation.restype = c.c_int
     L.glm_block_embedding.argtypes = [P, c.c_int32, c.c_int64, c.c_int32, P, c.c_int32, P, P]
     L.glm_block_embedding.restype = c.c_int
+    L.glm_bench_read.argtypes = [c.c_int, P, c.c_int32, c.c_int32, c.c_size_t, P, P]
+    L.glm_bench_read.restype = c.c_int
     L.glm_model_file_open.argtypes = [c.c_char_p, c.POINTER(P)]
     L.glm_model_file_open.restype = c.c_int
     L.glm_model_file_close.argtypes = [P]

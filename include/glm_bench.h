@@ -1,0 +1,33 @@
+/*
+ * Measurement aids of libglm_attn.so for `bench.py --ceiling`.  They have no counterpart in the reference
+ * and are no part of the attention path: kernels that only load, shaped like a launch of the decode
+ * kernel, so that the read rate this GPU gives such a launch can be measured beside the kernel's own.
+ */
+#ifndef GLM_BENCH_H
+#define GLM_BENCH_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum glm_bench_pattern {
+    GLM_BENCH_READ_LINEAR = 0,         /* one layer's caches (2 kv_heads cache_rows 128 halfs) in address order */
+    GLM_BENCH_READ_DECODE_PATTERN = 1, /* the same bytes as the decode kernel asks for them: K rows, V columns */
+    GLM_BENCH_READ_STREAM = 2,         /* `bytes` bytes in one long launch */
+    GLM_BENCH_EMPTY = 3                /* a launch of 256 workgroups that does nothing */
+};
+
+/* Launches one read kernel on `stream` (hipStream_t).  For patterns 0 and 1 `base` is a device buffer laid
+   out like one layer's caches ([kv_heads][cache_rows][128] then [kv_heads][128][cache_rows], fp16), cache_rows
+   a multiple of 256, and `bytes` its size; one workgroup of 8 waves per 256 cache rows and KV head.
+   `sink` is a device float that is never written in practice.  Returns a glm_attn status. */
+int glm_bench_read(int pattern, const void *base, int32_t cache_rows, int32_t kv_heads, size_t bytes, float *sink,
+                   void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* GLM_BENCH_H */
