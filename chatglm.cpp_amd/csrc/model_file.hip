@@ -257,9 +257,18 @@ int parse(glm_model_file *f) {
         }
         if (t.ne[0] % block_elems != 0) {
             return fail(GLM_ATTN_EINVAL, "model file is broken (tensor %s: row of %lld elements in blocks of %lld)",
-                        t.name.c_str(), (long long)t.ne[0], (long long)block_elems);
+                        printable(t.name).c_str(), (long long)t.ne[0], (long long)block_elems);
         }
-        t.nbytes = t.ne[0] / block_elems * block_bytes * t.ne[1] * t.ne[2] * t.ne[3];  // ggml_nbytes, contiguous
+        // ggml_nbytes of a contiguous tensor.  Every factor comes from the file: a product that does not
+        // fit 63 bits must not wrap into a size that passes the check against the mapping below.
+        t.nbytes = t.ne[0] / block_elems;
+        bool overflow = __builtin_mul_overflow(t.nbytes, block_bytes, &t.nbytes);
+        for (int i = 1; i < 4; i++) {
+            overflow = overflow || __builtin_mul_overflow(t.nbytes, t.ne[i], &t.nbytes);
+        }
+        if (overflow) {
+            return fail(GLM_ATTN_EINVAL, "model file is broken (tensor %s: bad shape)", printable(t.name).c_str());
+        }
         t.offset = (int64_t)((cur.pos + 15) & ~(size_t)15);                            // chatglm.cpp:381-382
         if ((size_t)t.offset > cur.size || (size_t)t.nbytes > cur.size - (size_t)t.offset) {
             return fail(GLM_ATTN_EINVAL, "model file is truncated (data of tensor %s)", printable(t.name).c_str());

@@ -126,7 +126,9 @@ class Pair:
 
     # ---- one call through both implementations
     def forward(self, layer, qkv, n_past, pos=None, mask=None, host_pos=False, entry="forward", n_ctx=None,
-                oracle_rows=None, use_default_mask=True):
+                oracle_rows=None, use_default_mask=True, row_pad=0):
+        """row_pad > 0: the device copy of qkv gets that many floats of NaN behind every row and the call is
+        made with qkv_row_stride = width + row_pad (entries "forward", "prefill" and "rope_append")."""
         torch = self.torch
         qlen = qkv.shape[0]
         if pos is None:
@@ -142,7 +144,14 @@ class Pair:
             orc.append(self.ocfg, qkv_ref, n_past, self.ref_k[layer], self.ref_v[layer])
             ref = orc.attend(self.ocfg, qkv_ref, n_past, self.ref_k[layer], self.ref_v[layer], attention_mask=mask,
                              rows=oracle_rows)
-        qkv_d = torch.from_numpy(qkv).to(self.dev)
+        stride = 0
+        if row_pad:
+            padded = np.full((qlen, self.width + row_pad), np.nan, dtype=np.float32)
+            padded[:, :self.width] = qkv
+            qkv_d = torch.from_numpy(padded).to(self.dev)
+            stride = self.width + row_pad
+        else:
+            qkv_d = torch.from_numpy(qkv).to(self.dev)
         pos_d = torch.from_numpy(np.ascontiguousarray(pos, dtype=np.int32)).to(self.dev)
         mask_d = None if mask is None else torch.from_numpy(np.ascontiguousarray(mask, dtype=np.float32)).to(self.dev)
         out_d = torch.full((qlen, self.h * self.d), float("nan"), dtype=torch.float32, device=self.dev)
@@ -150,7 +159,10 @@ class Pair:
         if entry == "forward":
             st = self.ctx.forward(layer, qkv_d.data_ptr(), qlen, n_past, out_d.data_ptr(),
                                   position_ids_ptr=None if host_pos else pos_d.data_ptr(),
-                                  position_ids_host=pos if host_pos else None, attention_mask_ptr=mp)
+                                  position_ids_host=pos if host_pos else None, attention_mask_ptr=mp,
+                                  qkv_row_stride=stride)
+        elif entry == "rope_append":  # the first half alone: caches only, no output
+            st = self.ctx.rope_append(layer, qkv_d.data_ptr(), pos_d.data_ptr(), qlen, n_past, qkv_row_stride=stride)
         elif entry == "decode":
             st = self.ctx.decode(layer, qkv_d.data_ptr(), n_past, out_d.data_ptr(),
                                  position_ids_ptr=None if host_pos else pos_d.data_ptr(),
@@ -161,7 +173,7 @@ class Pair:
                                         position_ids_host=pos if host_pos else None)
         elif entry == "prefill":
             st = self.ctx.prefill(layer, qkv_d.data_ptr(), pos_d.data_ptr(), qlen, n_past, out_d.data_ptr(),
-                                  attention_mask_ptr=mp)
+                                  attention_mask_ptr=mp, qkv_row_stride=stride)
         else:
             raise ValueError(entry)
         pkg.check(st, f"glm_attn_{entry}")

@@ -137,3 +137,17 @@ def test_library_exports_every_symbol_of_the_model_file_header():
     assert sorted(pkg.MODEL_FILE_SYMBOLS) == names
     assert lib.glm_model_file_open(None, None) == pkg.EINVAL
     assert lib.glm_block_embedding(None, 1, 8, 8, None, 1, None, None) == pkg.EINVAL
+
+
+def test_decode_launch_stamps_on_the_host(tmp_path):
+    """tests/cpp/test_decode_stamp.cpp: the stamp arithmetic of the decode kernel's exchange, compiled for the
+    host from the kernel's own header (a stamp is never 0, the count skips the one that would be)."""
+    import subprocess
+
+    exe = str(tmp_path / "test_decode_stamp")
+    src = os.path.join(ROOT, "tests", "cpp", "test_decode_stamp.cpp")
+    inc = ["-I" + os.path.join(ROOT, "include"), "-I" + os.path.join(ROOT, "chatglm.cpp_amd", "csrc")]
+    subprocess.run(["/opt/rocm/bin/hipcc", "-O1", "-std=c++17", "-x", "hip", "--offload-arch=gfx950", src, "-o", exe] + inc,
+                   check=True, capture_output=True)
+    out = subprocess.run([exe], capture_output=True, text=True)
+    assert out.returncode == 0 and out.stdout.strip() == "ok", out.stdout + out.stderr

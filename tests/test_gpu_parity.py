@@ -223,6 +223,25 @@ def test_position_out_of_table_sets_flag(H):
     p.close()
 
 
+@pytest.mark.parametrize("entry", ["forward", "prefill", "rope_append"])
+@pytest.mark.parametrize("interleaved,kvh,rope_type", [(False, 2, None), (True, 32, "glm1")])
+def test_padded_qkv_rows(H, entry, interleaved, kvh, rope_type):
+    """qkv_row_stride > width: the rows of the fused projection are views into a wider buffer (the views of
+    chatglm.cpp:636-653 carry their own row stride); what lies between the rows is NaN here."""
+    kw = dict(kvh=kvh, max_length=512, interleaved=interleaved)
+    if rope_type == "glm1":
+        kw.update(rope_type=H.orc.ROPE_CHATGLM, mask_type=H.orc.MASK_CHATGLM)
+    p = H.Pair(**kw)
+    p.fill_past(0, 100, seed=3)
+    for qlen, n_past in ((37, 100), (5, 137)):
+        qkv = p.random_qkv(qlen, seed=40 + qlen)
+        out, ref, _ = p.forward(0, qkv, n_past, entry=entry, row_pad=24, n_ctx=300)
+        p.assert_caches_equal(0, f"{entry} with padded rows")
+        if entry != "rope_append":
+            H.assert_close(out, ref, f"{entry} with padded rows, qlen {qlen}")
+    p.close()
+
+
 def test_range_errors(H):
     p = H.Pair(max_length=64)
     import torch

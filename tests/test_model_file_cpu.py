@@ -145,6 +145,13 @@ def test_broken_files_are_errors_with_the_reference_messages(tmp_path):
         hdr = f.config().tokenizer_offset + f.config().tokenizer_size
     struct.pack_into("i", bad_dims, hdr + 4 + name_len, 5)  # ndim = 5 (chatglm.cpp:371)
     assert "dimensions" in open_error(bytes(bad_dims))
+    # a shape whose byte count does not fit 64 bits must not wrap into a size that fits the file:
+    # 4 dims of 2^31 - 1 fp32 elements = 2^126 bytes (2^62 elements would wrap to a small count)
+    rec = struct.pack("i", 1) + b"w" + struct.pack("i" * 6, 4, 0x7fffffff, 0x7fffffff, 0x7fffffff, 0x7fffffff, 0)
+    assert "bad shape" in open_error(blob[:hdr] + rec + b"\0" * 64)
+    # 2^31-1 * 2^31-1 * 2 * 2 elements of fp16: 2^65 bytes, which is 2^1 modulo 2^64
+    rec = struct.pack("i", 1) + b"w" + struct.pack("i" * 6, 4, 0x40000000, 0x40000000, 4, 2, 1)
+    assert "bad shape" in open_error(blob[:hdr] + rec + b"\0" * 64)
 
 
 def test_mutated_files_never_crash_the_reader(tmp_path):
