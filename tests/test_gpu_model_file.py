@@ -36,11 +36,14 @@ def read_logits(path):
     return out
 
 
-def run_case(tmp_path, model_type, cfg, config_bytes, tensors, ids, n_prompt, all_rows, max_length=-1, tol=4e-3):
+def run_case(tmp_path, model_type, cfg, config_bytes, tensors, ids, n_prompt, all_rows, max_length=-1, tol=4e-3,
+             path=None):
+    """path: an existing model file that holds `tensors` (else one is written in the converter's layout)."""
     from model_host import OracleModel
 
-    path = str(tmp_path / "model.bin")
-    mw.write_model_file(path, model_type, config_bytes, b"tokenizer bytes", tensors)
+    if path is None:
+        path = str(tmp_path / "model.bin")
+        mw.write_model_file(path, model_type, config_bytes, b"tokenizer bytes", tensors)
     out_path = str(tmp_path / "logits.bin")
     print("running", os.path.basename(RUNNER), "model_type", model_type, flush=True)
     r = subprocess.run([RUNNER, path, out_path, str(max_length), str(n_prompt), str(int(all_rows))] + [str(i) for i in ids],
@@ -146,3 +149,19 @@ def test_a_prompt_of_more_than_8_tokens_takes_the_expanded_weights(tmp_path):
     tensors = mw.random_state_dict(GLM4, mw.glm2_weight_names(3), mw.glm2_shapes, 41, 8)
     ids = list(range(20, 32)) + [5, 6]
     run_case(tmp_path, 4, GLM4, mw.pack_config_v2(8, **GLM4), tensors, ids, 12, False, max_length=32, tol=4e-2)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("fname", ["glm2_f16", "glm3_ptuning_f16", "glm4_q8_0", "glm1_q5_1", "glm2_q4_0"])
+def test_files_written_by_the_reference_converter_run_end_to_end(tmp_path, fname):
+    """tests/golden/reference_converter/*.bin are bytes of chatglm_cpp/convert.py itself (see
+    tests/golden/make_model_file_goldens.py): loaded by the C++ model classes, run on the device, compared with the
+    oracle-composed model built from the tensors that went into the converter."""
+    import test_reference_converter_goldens as gold
+
+    _, sname, model_type, wtype, cfg, _ = next(f for f in gold.FILES if f[0] == fname)
+    state = np.load(os.path.join(gold.GOLD, sname + ".npz"))
+    tensors = gold.expected_tensors(state, model_type, wtype, cfg)
+    tol = 4e-3 if wtype in ("f16", "f32") else 4e-2
+    run_case(tmp_path, model_type, cfg, None, tensors, [3, 17, 30, 22, 9, 1], 3, False, tol=tol,
+             path=os.path.join(gold.GOLD, fname + ".bin"))

@@ -3,9 +3,9 @@
 derives from them (chatglm.h:106-160), tensor records with their 16-byte alignment (chatglm.cpp:357-391), and the
 checks on broken files.  No GPU: everything up to the upload is host code.
 
-Parity unpinned for the byte layout: the reference ships no model file to read, so the writer used here restates
-the converter's source and the reader restates the loader's; the two agree with each other and with both sources,
-which is all that can be shown without a checkpoint."""
+The reference ships no model file to read; the byte layout is pinned by tests/test_reference_converter_goldens.py,
+where the writer used here reproduces files of the reference's own converter byte for byte and the reader parses
+them."""
 import os
 import struct
 import sys
