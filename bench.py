@@ -364,7 +364,7 @@ def main():
                                     "peak": HBM_PEAK_GBS, "unit": "GB/s",
                                     "frac": round(bytes1 / ms1 / 1e6 / HBM_PEAK_GBS, 4), "bytes_per_layer": bytes1},
                 "prefill_ms_per_layer": round(msp, 4),
-                "prefill_roofline": {"bound": "mfma", "kernel": "hipBLASLt fp16 GEMM after round_rows_kernel", "achieved": round(flop_p / msp / 1e9, 1),
+                "prefill_roofline": {"bound": "mfma", "kernel": "gemm_f16_kernel after round_rows_kernel", "achieved": round(flop_p / msp / 1e9, 1),
                                      "peak": MFMA_FP16_PEAK_TFLOPS, "unit": "TFLOP/s",
                                      "frac": round(flop_p / msp / 1e9 / MFMA_FP16_PEAK_TFLOPS, 4),
                                      "rows": PREFILL_Q, "flops_per_layer": flop_p},

@@ -81,6 +81,7 @@ class LinearDesc(ctypes.Structure):
         ("device", ctypes.c_int32),
         ("weight", ctypes.c_void_p),
         ("bias", ctypes.c_void_p),
+        ("weight_bytes", ctypes.c_int64),
     ]
 
 
@@ -345,12 +346,12 @@ class Context:
 
 
 def make_linear_desc(in_features, out_features, weight_dtype=LINEAR_F16, use_bias=True, max_rows=1, device=0,
-                     weight=None, bias=None):
+                     weight=None, bias=None, weight_bytes=0):
     d = LinearDesc()
     d.struct_size = ctypes.sizeof(LinearDesc)
     d.in_features, d.out_features = in_features, out_features
     d.weight_dtype, d.use_bias, d.max_rows, d.device = weight_dtype, int(bool(use_bias)), max_rows, device
-    d.weight, d.bias = weight, bias
+    d.weight, d.bias, d.weight_bytes = weight, bias, weight_bytes
     return d
 
 

@@ -365,23 +365,12 @@ __global__ void gated_rows_f16_kernel(const float *x, const float *up, int activ
     }
 }
 
-// y += residual * scale, for the GEMM that cannot take the residual itself
-__global__ void add_residual_kernel(float *y, const float *residual, float scale, int64_t n4) {
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += (int64_t)gridDim.x * blockDim.x) {
-        floatx4 v = *reinterpret_cast<const floatx4 *>(y + i * 4);
-        const floatx4 r = *reinterpret_cast<const floatx4 *>(residual + i * 4);
-#pragma unroll
-        for (int e = 0; e < 4; e++) {
-            v[e] = __fadd_rn(v[e], __fmul_rn(r[e], scale));
-        }
-        *reinterpret_cast<floatx4 *>(y + i * 4) = v;
-    }
-}
-
 // Y^T tile = W tile (features on MFMA rows) x X^T tile (input rows on MFMA columns).  Waves: 2 x 2, each
 // 64 features x 64 input rows = 2 x 2 blocks of 32 x 32.
+// `residual` (or null) has y's shape and may be y itself: a lane reads its 4 values right before it writes the same 4.
 __global__ __launch_bounds__(GM_THREADS, 2) void gemm_f16_kernel(const __half *W, const float *bias, const __half *x16,
-                                                                 int rows, int K, int N, float *y) {
+                                                                 int rows, int K, int N, float *y, const float *residual,
+                                                                 float residual_scale) {
     __shared__ __attribute__((aligned(1024))) __half Ws[2][GM_TILE][GM_K];
     __shared__ __attribute__((aligned(1024))) __half Xs[2][GM_TILE][GM_K];
     const int tid = threadIdx.x, lane = tid & 63;
@@ -448,6 +437,13 @@ __global__ __launch_bounds__(GM_THREADS, 2) void gemm_f16_kernel(const __half *W
                                      acc[fb][rb][4 * b4 + 3]};
                         if (bias) {
                             v += *reinterpret_cast<const floatx4 *>(bias + f);
+                        }
+                        if (residual) {
+                            const floatx4 r = *reinterpret_cast<const floatx4 *>(residual + (int64_t)row * N + f);
+#pragma unroll
+                            for (int e = 0; e < 4; e++) {
+                                v[e] = __fadd_rn(v[e], __fmul_rn(r[e], residual_scale));
+                            }
                         }
                         *reinterpret_cast<floatx4 *>(y + (int64_t)row * N + f) = v;
                     }
@@ -584,11 +580,13 @@ void free_linear(glm_linear *l) {
     delete l;
 }
 
-// The device's handle and workspace; null if hipBLASLt cannot be set up (the library's own GEMM is used then).
+// The device's hipBLASLt handle and workspace, or null: then the library's own GEMM kernel runs, which is the
+// default.  hipBLASLt is used only when the environment holds GLM_LINEAR_HIPBLASLT=1 at glm_linear_create: two
+// timing programs that drove many-row calls through it ended in GPU memory faults whose cause was never shown.
 LtDevice *lt_device(int device) {
     if (device < 0 || device >= 64) return nullptr;
-    const char *own = getenv("GLM_LINEAR_OWN_GEMM");  // set to 1 to run the library's own GEMM kernel instead
-    if (own && own[0] == '1') return nullptr;
+    const char *lt = getenv("GLM_LINEAR_HIPBLASLT");
+    if (!lt || lt[0] != '1') return nullptr;
     std::lock_guard<std::mutex> lock(g_lt_mutex);
     LtDevice &d = g_lt[device];
     if (!d.handle) {
@@ -653,7 +651,7 @@ LtPlan *lt_plan(glm_linear *l, int rows) {
                     HIPBLAS_STATUS_SUCCESS &&
                 hipblasLtMatmulAlgoGetHeuristic(l->lt->handle, l->lt_desc, l->lt_la, p.lb, p.lc, p.lc, pref, 1, &res,
                                                 &found) == HIPBLAS_STATUS_SUCCESS &&
-                found > 0) {
+                found > 0 && res.state == HIPBLAS_STATUS_SUCCESS && res.workspaceSize <= ws) {
                 p.algo = res.algo;
                 p.usable = true;
             }
@@ -676,6 +674,10 @@ int glm_linear_create(const glm_linear_desc *desc, glm_linear **out_linear) {
     if (quant && desc->in_features % 32 != 0) return GLM_ATTN_EINVAL;  // ggml's blocks hold 32 inputs
     if (quant && (desc->device < 0 || desc->device >= 64)) return GLM_ATTN_EINVAL;
     if (!desc->use_bias && desc->bias) return GLM_ATTN_EINVAL;
+    if (desc->weight_bytes < 0 || (desc->weight_bytes > 0 && !desc->weight)) return GLM_ATTN_EINVAL;
+    if (desc->weight && desc->weight_bytes > 0 && (uint64_t)desc->weight_bytes < (uint64_t)weight_bytes(*desc)) {
+        return GLM_ATTN_EINVAL;  // the kernels would read past the caller's allocation
+    }
     if (hipSetDevice(desc->device) != hipSuccess) return GLM_ATTN_EHIP;
     glm_linear *l = new (std::nothrow) glm_linear();
     if (!l) return GLM_ATTN_ENOMEM;
@@ -871,6 +873,9 @@ static int linear_forward_impl(glm_linear *l, glm_linear *l2, const glm_linear_f
         (!gemv || (pro == GLM_LINEAR_PRO_RMS_NORM && (int64_t)rows * ((K / 32 + GV_WAVES - 1) / GV_WAVES) > 32))) {
         return GLM_ATTN_EUNSUPPORTED;
     }
+    // the shared per-device buffers hold what this call writes into them (they only grow, at glm_linear_create)
+    if (gemm && sizeof(__half) * (size_t)rows * (size_t)K > l->staging->bytes) return GLM_ATTN_ERANGE;
+    if (need_dequant && sizeof(__half) * (size_t)N * (size_t)K > l->dequant->bytes) return GLM_ATTN_ERANGE;
     if (need_dequant) {
         launch_dequant_f16(l->q, l->dequant->x16, stream);
     }
@@ -955,12 +960,7 @@ static int linear_forward_impl(glm_linear *l, glm_linear *l2, const glm_linear_f
         if (!done) {
             hipLaunchKernelGGL(gemm_f16_kernel, dim3((N + GM_TILE - 1) / GM_TILE, (rows + GM_TILE - 1) / GM_TILE),
                                dim3(GM_THREADS), 0, stream, static_cast<const __half *>(weight), l->bias, l->staging->x16,
-                               rows, K, N, y);
-            if (residual) {
-                const int64_t o4 = (int64_t)rows * N / 4;
-                const int rb = (int)((o4 + 255) / 256 < 2048 ? (o4 + 255) / 256 : 2048);
-                hipLaunchKernelGGL(add_residual_kernel, dim3(rb), dim3(256), 0, stream, y, residual, fu->residual_scale, o4);
-            }
+                               rows, K, N, y, residual, residual ? fu->residual_scale : 0.f);
         }
     } else {
         const int64_t n_out = (int64_t)rows * N;

@@ -182,7 +182,7 @@ int main(int argc, char **argv) {
         double prefill_ms = 0.0;
         if (prompt > 0) {
             std::vector<int> seen(ids.begin(), ids.begin() + prompt);
-            model.forward_graph_compute(seen, 0, prompt, true);  // warm-up: arenas grow, hipBLASLt picks its algorithms
+            model.forward_graph_compute(seen, 0, prompt, true);  // warm-up: arenas grow
             const double t0 = now_ms();
             std::vector<float> logits = model.forward_graph_compute(seen, 0, prompt, true);
             prefill_ms = now_ms() - t0;

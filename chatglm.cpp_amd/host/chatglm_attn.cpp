@@ -208,6 +208,7 @@ Linear::Linear(ModelContext *mctx, int in_features, int out_features, bool use_b
                       tied_weight->ne[1] == out_features && tied_weight->data)
             << "tied weight must be an allocated [out_features, in_features] tensor of the context's dtype";
         desc.weight = tied_weight->data;
+        desc.weight_bytes = (int64_t)tied_weight->nbytes();
     }
     glm_linear *raw = nullptr;
     CHATGLM_CHECK_ATTN(glm_linear_create(&desc, &raw));

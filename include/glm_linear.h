@@ -20,9 +20,10 @@
  * expansion goes into one buffer per device, as large as the largest quantised weight created on it: such calls
  * on one device must not overlap on different streams.
  *
- * Calls with more than 8 rows are plain GEMMs and go to hipBLASLt (fp16 x fp16, fp32 accumulation and output, bias
- * epilogue) after the rows have been rounded; for shapes hipBLASLt has no algorithm for, or with
- * GLM_LINEAR_OWN_GEMM=1 in the environment when the layer is created, the library's own MFMA GEMM runs instead.
+ * Calls with more than 8 rows are plain GEMMs (fp16 x fp16, fp32 accumulation and output) on the library's own MFMA
+ * kernel after the rows have been rounded.  With GLM_LINEAR_HIPBLASLT=1 in the environment when the layer is created
+ * they go to hipBLASLt instead (bias epilogue; the own kernel for shapes it has no algorithm for): faster, but off
+ * by default, because two timing programs that drove it ended in GPU memory faults whose cause was never shown.
  *
  * All pointers named "device" are HIP device pointers; calls are asynchronous on the given stream.  Status
  * codes are those of glm_attn.h (0 = ok, negative = error; glm_attn_strerror names them).
@@ -66,6 +67,9 @@ typedef struct glm_linear_desc {
                              ggml blocks); NULL: the library allocates (zero-filled) and the caller fills it
                              through glm_linear_params */
     float *bias;          /* optional caller-owned device tensor [out_features]; NULL: as for weight */
+    int64_t weight_bytes; /* bytes the caller's allocation holds from `weight` on, or 0 if not stated (and with a NULL
+                             weight): a value below out_features x in_features elements (quantised types: blocks) is
+                             refused with GLM_ATTN_EINVAL before any device call */
 } glm_linear_desc;
 
 /* Linear::Linear (chatglm.h:365-367). */

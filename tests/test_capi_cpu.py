@@ -100,6 +100,16 @@ def test_bad_linear_descriptors_are_rejected_without_a_device():
     assert pkg.lib().glm_linear_create(ctypes.byref(d), ctypes.byref(h)) == pkg.EUNSUPPORTED
     d = pkg.make_linear_desc(48, 32, weight_dtype=8)  # GGML_TYPE_Q8_0 holds blocks of 32 inputs
     assert pkg.lib().glm_linear_create(ctypes.byref(d), ctypes.byref(h)) == pkg.EINVAL
+    # a caller-owned weight whose stated allocation is shorter than what the kernels read (64 x 32 fp16 = 4096 B;
+    # Q8_0: 2 blocks of 34 B per feature) is refused before any device call; a size without a weight as well
+    d = pkg.make_linear_desc(64, 32, weight=0x1000, weight_bytes=4095)
+    assert pkg.lib().glm_linear_create(ctypes.byref(d), ctypes.byref(h)) == pkg.EINVAL
+    d = pkg.make_linear_desc(64, 32, weight_dtype=8, weight=0x1000, weight_bytes=32 * 2 * 34 - 1)
+    assert pkg.lib().glm_linear_create(ctypes.byref(d), ctypes.byref(h)) == pkg.EINVAL
+    d = pkg.make_linear_desc(64, 32, weight_bytes=4096)
+    assert pkg.lib().glm_linear_create(ctypes.byref(d), ctypes.byref(h)) == pkg.EINVAL
+    d = pkg.make_linear_desc(64, 32, weight=0x1000, weight_bytes=-1)
+    assert pkg.lib().glm_linear_create(ctypes.byref(d), ctypes.byref(h)) == pkg.EINVAL
     assert pkg.lib().glm_linear_commit(None, None) == pkg.EINVAL
     assert pkg.lib().glm_linear_forward(None, None, 1, None, None) == pkg.EINVAL
 
