@@ -14,6 +14,24 @@
 
 namespace glm_attn {
 
+#ifdef GLM_ATTN_TIMELINE
+// Instrumented build: every wave of prefill_kernel leaves 100 MHz clock readings here.
+__device__ unsigned long long g_prefill_timeline[kTimelineSlots * 16];
+#define PTS(i)                                                                                                   \
+    do {                                                                                                         \
+        const int slot_ = (blockIdx.y * gridDim.x + blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6);        \
+        if ((threadIdx.x & 63) == 0 && slot_ < kTimelineSlots) g_prefill_timeline[slot_ * 16 + (i)] = wall_clock64(); \
+    } while (0)
+extern "C" int glm_attn_debug_prefill_timeline(unsigned long long *host, size_t n) {
+    if (n > (size_t)kTimelineSlots * 16) n = (size_t)kTimelineSlots * 16;
+    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(g_prefill_timeline), n * sizeof(unsigned long long));
+}
+#else
+#define PTS(i) \
+    do {       \
+    } while (0)
+#endif
+
 namespace {
 
 constexpr int D = kFastHeadSize;
@@ -25,6 +43,18 @@ constexpr float LOG2E = 1.4426950408889634f;
 constexpr int kPrefillMaxSplits = 128;
 constexpr int RING = 3;  // LDS fragments in flight ahead of the MFMAs (4 no longer fit the 256 registers)
 constexpr float kLazy = 8.f;  // see the online softmax in the kernel
+
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+
+// maximum / sum of a value over lane i and lane i ^ 32 (v_permlane32_swap: no trip through LDS)
+__device__ inline float max_of_halves(float x) {
+    const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
+}
+__device__ inline float sum_of_halves(float x) {
+    const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
+}
 
 __device__ inline floatx16 mfma32(half8 a, half8 b, floatx16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
@@ -98,6 +128,7 @@ __device__ inline uint32_t v_offset_clamped(int L, int w, int lane, int left) {
 }
 
 // V columns of keys that do not exist (>= kvs) may hold anything, and 0 * NaN is NaN: zero them in LDS.
+// (tid: 0..THREADS-1 within the four waves that own the buffer)
 __device__ inline void zero_missing_columns(__half (*Vs)[BN], int key0, int kvs, int tid) {
     asm volatile("" : "+v"(tid));  // rare path: keeps its index arithmetic from being hoisted out of the tile loop
     for (int idx = tid; idx < D * BN; idx += THREADS) {
@@ -117,18 +148,32 @@ __device__ inline void zero_missing_columns(__half (*Vs)[BN], int key0, int kvs,
 //
 // order: how workgroup ids map to (token tile, head) items.  0: tile-major as they come (all items
 // cost the same).  Causal items cost more the later their tile: 1 starts the longest first, which
-// lets the dispatcher even the slots out when there are several rounds of workgroups; 2, for a grid
-// that fits the chip in one round of two per CU, also puts the i-th longest and the i-th shortest half
-// a grid apart, which is where the two workgroups of a CU come from.
-__global__ __launch_bounds__(THREADS, 2) void prefill_kernel(AttendArgs a, int n_qtiles, int order, int packed) {
-    // K tiles [2][BN][D], then V tiles [2][D][BN]; tile T of either lives in buffer T & 1
-    __shared__ __attribute__((aligned(1024))) __half smem[2 * BN * D + 2 * D * BN];
-    const uint32_t smem_at = (uint32_t)reinterpret_cast<uintptr_t>(&smem[0]);  // LDS byte address
+// lets the dispatcher even the slots out; 2, for a grid that fills the chip exactly once with two workgroups
+// per CU, also puts the i-th longest and the i-th shortest half a grid apart, which is where the two
+// workgroups of a CU come from.
+//
+// GROUPS: 1, or 2 for a grid with too few workgroups to give every CU two of them (a prompt of a few thousand
+// tokens or less).  Then a workgroup has eight waves in two groups of four that own the same 128 rows; each group
+// is what a whole workgroup is otherwise, with its own tile buffers, and takes every other tile of the key range;
+// the second group hands its (m, l, O) to the first through LDS at the end.  A CU then holds its eight waves on
+// one item at a time: no tail in which the long item of a causal prompt runs alone at half the occupancy, and no
+// pass over partial results in global memory.
+template <int GROUPS>
+__global__ __launch_bounds__(THREADS * GROUPS, 2 / GROUPS) void prefill_kernel(AttendArgs a, int n_qtiles, int order,
+                                                                              int packed) {
+    // per group: K tiles [2][BN][D], then V tiles [2][D][BN]; the k-th tile of a group lives in buffer k & 1
+    constexpr int GROUP_HALFS = 2 * BN * D + 2 * D * BN;
+    __shared__ __attribute__((aligned(1024))) __half smem_all[GROUPS * GROUP_HALFS];
     constexpr uint32_t TILE_BYTES = BN * D * 2;  // a K tile and a V tile are the same size
     constexpr uint32_t V_AT = 2 * TILE_BYTES;
 
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);  // in a scalar register: LDS targets of the copy are per wave
+    PTS(0);
+    const int lane = threadIdx.x & 63;
+    const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // in a scalar register: LDS targets of the copy are per wave
+    const int grp = GROUPS > 1 ? wv >> 2 : 0, w = wv & 3;
+    const int tid = threadIdx.x & (THREADS - 1);  // within the group
+    __half *const smem = smem_all + grp * GROUP_HALFS;
+    const uint32_t smem_at = (uint32_t)reinterpret_cast<uintptr_t>(smem);  // LDS byte address
     const int n = lane & 31, c = lane >> 5;
     // A workgroup owns 128 rows of one unit.  Normally a unit is a query head and its rows are the tokens.
     // packed: a unit is a KV group and its rows are (head of the group, token) pairs, head-major, so that a
@@ -137,10 +182,9 @@ __global__ __launch_bounds__(THREADS, 2) void prefill_kernel(AttendArgs a, int n
     const int heads_per_unit = packed ? a.s.G : 1;
     const int units = a.s.h / heads_per_unit;
     const int rows = heads_per_unit * a.qlen;
-    const int n_items = n_qtiles * units;
     int item = blockIdx.x;
-    if (order == 2 && item >= n_items / 2) {
-        item = n_items - 1 - (item - n_items / 2);
+    if (order == 2 && item >= (int)gridDim.x / 2) {
+        item = (int)gridDim.x - 1 - (item - (int)gridDim.x / 2);
     }
     const int qt = order ? n_qtiles - 1 - item / units : item / units;
     const int unit = item % units;
@@ -200,10 +244,13 @@ __global__ __launch_bounds__(THREADS, 2) void prefill_kernel(AttendArgs a, int n
         }
         return;
     }
-    // The loop below is written for two tiles per round (the two score accumulators swap roles); an odd
-    // count is rounded up with a tile whose keys are all masked.  Copies of tiles past the last one read
-    // the last one again.
-    const int n_iter = (t1 - t0 + 1) & ~1;
+    // The loop below is written for two tiles per round (the two score accumulators swap roles), and every
+    // group runs the same number of rounds (they meet at the same barriers): group g takes tiles t0 + g,
+    // t0 + g + GROUPS, ...; what that reaches beyond the share are tiles whose keys are all masked (key >= kv_lim).
+    // Copies of tiles past the last one read the last one again.
+    const int n_iter = ((t1 - t0 + GROUPS - 1) / GROUPS + 1) & ~1;
+    const int tg0 = t0 + grp;  // this group's first tile
+    const int kv_lim = a.kvs < t1 * BN ? a.kvs : t1 * BN;
 
     const TileCopy tc = tile_copy_lanes(L, w, lane);
     // pieces 0..3 of the copy of K tile `tile` / V tile `tile` into buffer `buf`
@@ -222,11 +269,11 @@ __global__ __launch_bounds__(THREADS, 2) void prefill_kernel(AttendArgs a, int n
 
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-        copy_k(t0, i, 0);
+        copy_k(tg0, i, 0);
     }
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-        copy_k(t0 + 1, i, 1);
+        copy_k(tg0 + GROUPS, i, 1);
     }
     // the second product of the first iteration stands for a tile -1: probabilities 0 times V buffer 1,
     // which must hold finite numbers for that
@@ -236,7 +283,7 @@ __global__ __launch_bounds__(THREADS, 2) void prefill_kernel(AttendArgs a, int n
         for (int e = 0; e < 8; e++) {
             z[e] = (_Float16)0.f;
         }
-        reinterpret_cast<half8 *>(smem + 2 * BN * D + D * BN)[idx] = z;
+        reinterpret_cast<half8 *>(smem + 2 * BN * D + D * BN)[idx] = z;  // (the group's own buffer, its own threads)
     }
 
     // Q^T operand: token n, dims t*16 + c*8 .. +8, resident for the whole kernel
@@ -259,8 +306,15 @@ __global__ __launch_bounds__(THREADS, 2) void prefill_kernel(AttendArgs a, int n
             o[db][r] = 0.f;
         }
     }
-    float m = -INFINITY, l = 0.f;  // reference point of the exponentials (log2 units) and sum for token n
-    half8 pf[4];                   // probabilities of the tile whose second product comes next
+    // Reference point of the exponentials for token n (log2 units, the same in both lane halves) and the sum of
+    // the probabilities of this lane's keys (the two halves of a token are added up after the last tile).
+    float m = -INFINITY, l = 0.f;
+    floatx16 nb;  // -m in every register (0 while m is -inf): where the score sums start
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+        nb[r] = 0.f;
+    }
+    half8 pf[4];  // probabilities of the tile whose second product comes next
 #pragma unroll
     for (int ks = 0; ks < 4; ks++) {
 #pragma unroll
@@ -292,8 +346,10 @@ __global__ __launch_bounds__(THREADS, 2) void prefill_kernel(AttendArgs a, int n
         return *(lds_frag)(uintptr_t)(va[j >> 2] + (uint32_t)(buf * TILE_BYTES + (j & 3) * 32 * BN * 2));
     };
 
-    // S^T = K Q^T for the K tile in buffer buf: two 32-key blocks.  The 16 fragments come through a ring, so
-    // that a read is issued RING MFMAs before its use.  between(i) runs after step i.
+    // S^T = K Q^T - m for the K tile in buffer buf: two 32-key blocks.  The 16 fragments come through a ring, so
+    // that a read is issued RING MFMAs before its use.  between(i) runs after step i.  The sums start from
+    // nb, which holds minus the reference point of the exponentials in all its registers (the lane's token is the
+    // same for all of them): the scores leave the matrix pipe ready for v_exp_f32.
     auto first_product = [&](int buf, floatx16 (&s)[2], auto between) __attribute__((always_inline)) {
         half8 fr[RING];
 #pragma unroll
@@ -301,13 +357,8 @@ __global__ __launch_bounds__(THREADS, 2) void prefill_kernel(AttendArgs a, int n
             fr[i] = kfrag(buf, i);
         }
 #pragma unroll
-        for (int r = 0; r < 16; r++) {
-            s[0][r] = 0.f;
-            s[1][r] = 0.f;
-        }
-#pragma unroll
         for (int i = 0; i < 16; i++) {
-            s[i & 1] = mfma32(fr[i % RING], qf[i >> 1], s[i & 1]);
+            s[i & 1] = mfma32(fr[i % RING], qf[i >> 1], i < 2 ? nb : s[i & 1]);
             if (i + RING < 16) {
                 fr[i % RING] = kfrag(buf, i + RING);
             }
@@ -335,25 +386,32 @@ __global__ __launch_bounds__(THREADS, 2) void prefill_kernel(AttendArgs a, int n
 
     // The wait is the builtin, not assembly: the compiler then knows that its own loads (the queries) are
     // over too and puts no waits for them between the MFMAs, where they would wait for the copies.
+    PTS(1);
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
     __syncthreads();
+    PTS(2);
     first_product(0, sa, [](int) {});
+    PTS(3);
 
-    // One iteration: sc holds the scores of tile T (buffer parity par = T & 1), sn takes those of tile T+1.
+    // One iteration: sc holds the scores of tile T (in the buffers of parity par), sn takes those of the group's
+    // next tile.  In the comments T+1, T-1, ... count the group's own tiles (GROUPS apart in the key range).
     auto iteration = [&](const int T, const int par, floatx16 (&sc)[2], floatx16 (&sn)[2]) __attribute__((always_inline)) {
         const int key0 = T * BN;
         // K(T+1) and V(T-1) have landed for every wave, and nobody reads K(T) or V(T-2) any more
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
         __syncthreads();
-        if (T > t0 && key0 > a.kvs) {  // V(T-1) has columns past the end
-            zero_missing_columns(reinterpret_cast<__half (*)[BN]>(smem + 2 * BN * D + (par ^ 1) * D * BN), key0 - BN,
-                                 a.kvs, tid);
+        // V(T-1) has columns past the end, in this group or in another one (all groups take the barrier)
+        if (T != tg0 && (T - grp) * BN > a.kvs) {
+            if ((T - GROUPS + 1) * BN > a.kvs) {
+                zero_missing_columns(reinterpret_cast<__half (*)[BN]>(smem + 2 * BN * D + (par ^ 1) * D * BN),
+                                     (T - GROUPS) * BN, a.kvs, tid);
+            }
             __syncthreads();
         }
         const uint32_t tcv = v_lanes(T);
 
         // ---- mask
-        const bool need_mask = (key0 + BN > a.kvs) || (a.causal && key0 + BN - 1 > a.p0 + wave_t_min) || a.mask;
+        const bool need_mask = (key0 + BN > kv_lim) || (a.causal && key0 + BN - 1 > a.p0 + wave_t_min) || a.mask;
         if (need_mask) {
             int nn = n;
             asm volatile("" : "+v"(nn));  // so that the token is not worked out before the loop and kept
@@ -366,9 +424,9 @@ __global__ __launch_bounds__(THREADS, 2) void prefill_kernel(AttendArgs a, int n
                     const int key = key0 + kb * 32 + 16 * (b >> 1) + 8 * c + 4 * (b & 1) + (r & 3);
                     float v = sc[kb][r];
                     if (a.mask && key < a.kvs) {
-                        v += a.mask[(int64_t)t_abs * a.kvs + key];
+                        v = __builtin_fmaf(a.mask[(int64_t)t_abs * a.kvs + key], LOG2E, v);  // scores are in log2 units
                     }
-                    if (key >= a.kvs || (a.causal && key > a.p0 + t_abs)) {
+                    if (key >= kv_lim || (a.causal && key > a.p0 + t_abs)) {
                         v = -INFINITY;
                     }
                     sc[kb][r] = v;
@@ -388,7 +446,7 @@ __global__ __launch_bounds__(THREADS, 2) void prefill_kernel(AttendArgs a, int n
         // of the exponentials only moves when the running maximum has grown by more than kLazy (in log2
         // units): probabilities may then reach 2^kLazy, which fp16 holds with full relative precision, and
         // the rescaling of the 64 accumulator registers becomes rare.
-        float mx = -INFINITY;
+        float mx = -INFINITY;  // over the scores as they are: relative to m
 #pragma unroll
         for (int kb = 0; kb < 2; kb++) {
 #pragma unroll
@@ -396,61 +454,114 @@ __global__ __launch_bounds__(THREADS, 2) void prefill_kernel(AttendArgs a, int n
                 mx = fmaxf(mx, sc[kb][r]);
             }
         }
-        mx = fmaxf(mx, __shfl_xor(mx, 32));
-        const float m_cand = fmaxf(m, mx * LOG2E);
-        const bool move = (m_cand > m + kLazy) || (m == -INFINITY && m_cand != -INFINITY);
+        mx = max_of_halves(mx);
+        const bool move = (mx > kLazy) || (m == -INFINITY && mx != -INFINITY);
         second_product(par ^ 1, [&](int j) {
-            if ((j & 3) == 3) {
-                copy_k(T + 2, j >> 2, par);
+            if ((j & 3) == 1) {
+                copy_v(T, j >> 2, par, tcv);
+            } else if ((j & 3) == 3) {
+                copy_k(T + 2 * GROUPS, j >> 2, par);
             }
         });
         if (__builtin_amdgcn_ballot_w64(move) != 0) {
-            const float alpha = (m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m - m_cand);
+            // by how much the reference point rises (from 0 to the maximum for a token's first keys)
+            const float d = (mx == -INFINITY) ? 0.f : (m == -INFINITY ? mx : fmaxf(mx, 0.f));
+            const float alpha = (m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(-d);
 #pragma unroll
             for (int db = 0; db < 4; db++) {
                 o[db] *= alpha;
             }
             l *= alpha;
-            m = m_cand;
+            if (mx != -INFINITY) {
+                m = (m == -INFINITY) ? mx : m + d;
+            }
+            const float nm = (m == -INFINITY) ? 0.f : -m;
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                sc[0][r] -= d;  // this tile's scores were taken relative to the old point
+                sc[1][r] -= d;
+                nb[r] = nm;
+            }
         }
 
         // ---- first product of tile T+1, with the exponentials of tile T in its shadow and the copy of V(T)
-        const float m_ref = (m == -INFINITY) ? 0.f : m;
-        first_product(par ^ 1, sn, [&](int i) {
-            if ((i & 3) == 3) {
-                copy_v(T, i >> 2, par, tcv);
-            }
-        });
-        float psum = 0.f;
+        first_product(par ^ 1, sn, [](int) {});
+        // two probabilities per conversion; the sum is taken over the rounded values, the ones the second
+        // product multiplies (v_dot2_f32_f16 against ones: fp32 sums of pairs)
+        const half2v ones = {(_Float16)1.f, (_Float16)1.f};
 #pragma unroll
         for (int kb = 0; kb < 2; kb++) {
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[kb][r], LOG2E, -m_ref));
-                psum += p;
+            for (int r = 0; r < 16; r += 2) {
+                const half2v h = {(_Float16)__builtin_amdgcn_exp2f(sc[kb][r]), (_Float16)__builtin_amdgcn_exp2f(sc[kb][r + 1])};
+                l = __builtin_amdgcn_fdot2(h, ones, l, false);
                 const int b = r >> 2;
-                pf[kb * 2 + (b >> 1)][4 * (b & 1) + (r & 3)] = (_Float16)p;
+                pf[kb * 2 + (b >> 1)][4 * (b & 1) + (r & 3)] = h[0];
+                pf[kb * 2 + (b >> 1)][4 * (b & 1) + (r & 3) + 1] = h[1];
             }
         }
-        psum += __shfl_xor(psum, 32);
-        l += psum;
     };
 
-    for (int T = t0; T < t0 + n_iter; T += 2) {
+    for (int T = tg0; T < tg0 + n_iter * GROUPS; T += 2 * GROUPS) {
         iteration(T, 0, sa, sb);
-        iteration(T + 1, 1, sb, sa);
+        if (T == tg0) PTS(8);
+        iteration(T + GROUPS, 1, sb, sa);
+        if (T == tg0) PTS(9);
+        if (T == tg0 + 2 * GROUPS) PTS(10);
     }
+    PTS(4);
 
     // ---- second product of the last tile (n_iter is even: V buffer 1)
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
     __syncthreads();
-    if ((t0 + n_iter) * BN > a.kvs) {
-        zero_missing_columns(reinterpret_cast<__half (*)[BN]>(smem + 2 * BN * D + D * BN), (t0 + n_iter - 1) * BN, a.kvs,
-                             tid);
+    if ((t0 + n_iter * GROUPS) * BN > a.kvs) {  // in some group
+        const int T_last = tg0 + (n_iter - 1) * GROUPS;
+        if ((T_last + 1) * BN > a.kvs) {
+            zero_missing_columns(reinterpret_cast<__half (*)[BN]>(smem + 2 * BN * D + D * BN), T_last * BN, a.kvs, tid);
+        }
         __syncthreads();
     }
     second_product(1, [](int) {});
+    PTS(5);
 
+    l = sum_of_halves(l);
+    if (GROUPS > 1) {
+        // ---- the second group's (m, l, O) into the first's: wave w of either holds the same rows in the same
+        // lanes, so O goes through LDS register by register, 64 lanes side by side (the second group's own tile
+        // buffers are exactly 4 waves x 64 registers x 64 lanes of fp32), m and l through the first group's.
+        __syncthreads();  // every wave has read its last tile
+        float *xo = reinterpret_cast<float *>(smem_all + GROUP_HALFS) + w * 64 * 64 + lane;
+        float *xml = reinterpret_cast<float *>(smem_all) + w * 128 + lane;
+        if (grp == 1) {
+#pragma unroll
+            for (int db = 0; db < 4; db++) {
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    xo[(db * 16 + r) * 64] = o[db][r];
+                }
+            }
+            xml[0] = m;
+            xml[64] = l;
+        }
+        __syncthreads();
+        if (grp == 1) {
+            return;
+        }
+        const float m1 = xml[0], l1 = xml[64];
+        const float M = fmaxf(m, m1);
+        const float a0 = (m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m - M);
+        const float a1 = (m1 == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m1 - M);
+#pragma unroll
+        for (int db = 0; db < 4; db++) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                o[db][r] = o[db][r] * a0 + xo[(db * 16 + r) * 64] * a1;
+            }
+        }
+        l = l * a0 + l1 * a1;
+        m = M;
+    }
+    PTS(6);
     // ---- out[t][head*128 + dim] = O / l, or this share's (m, l, O) as they are
     if (nsplit > 1 && c == 0) {
         float *ml = part_ml();
@@ -475,37 +586,31 @@ __global__ __launch_bounds__(THREADS, 2) void prefill_kernel(AttendArgs a, int n
             }
         }
     }
+    PTS(7);
 }
 
 // out[t][head] = sum_s O_s 2^(m_s - M) / sum_s l_s 2^(m_s - M) over the shares of the key range, M = max m_s.
-// One workgroup per (row, unit): 32 threads of four dims each, times 8 that take every eighth share.
+// 32 threads of four dims each per (row, unit), eight of those per workgroup; a thread walks the shares itself.
 __global__ __launch_bounds__(256) void merge_splits_kernel(AttendArgs a, int padded_rows, int nsplit, int packed) {
-    __shared__ float red_m[8];
-    __shared__ floatx4 red_o[8][D / 4];
-    __shared__ float red_l[8];
     const int heads_per_unit = packed ? a.s.G : 1;
     const int units = a.s.h / heads_per_unit;
-    const int r = blockIdx.x, unit = blockIdx.y;
+    const int rows = heads_per_unit * a.qlen;
+    const int64_t ru = (int64_t)blockIdx.x * 8 + (threadIdx.x >> 5);  // (row, unit) in the order of the partials
+    if (ru >= (int64_t)rows * units) {
+        return;
+    }
+    const int r = (int)(ru / units), unit = (int)(ru % units);
     const int t = r % a.qlen, hh = unit * heads_per_unit + r / a.qlen;
-    const int d4 = threadIdx.x & 31, part = threadIdx.x >> 5;
+    const int d4 = threadIdx.x & 31;
     const float *ml = a.split_scratch + (int64_t)nsplit * padded_rows * units * D;
     auto prow = [&](int sp) { return ((int64_t)sp * padded_rows + r) * units + unit; };
     float M = -INFINITY;
-    for (int sp = threadIdx.x; sp < nsplit; sp += 256) {
+    for (int sp = 0; sp < nsplit; sp++) {
         M = fmaxf(M, ml[prow(sp) * 2]);
     }
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
-        M = fmaxf(M, __shfl_xor(M, off));
-    }
-    if ((threadIdx.x & 63) == 0) {
-        red_m[threadIdx.x >> 6] = M;
-    }
-    __syncthreads();
-    M = fmaxf(fmaxf(red_m[0], red_m[1]), fmaxf(red_m[2], red_m[3]));
     floatx4 acc = {0.f, 0.f, 0.f, 0.f};
     float lsum = 0.f;
-    for (int sp = part; sp < nsplit; sp += 8) {
+    for (int sp = 0; sp < nsplit; sp++) {
         const float *rec = ml + prow(sp) * 2;
         if (rec[1] == 0.f) {
             continue;  // a share without keys left its O unwritten
@@ -514,19 +619,7 @@ __global__ __launch_bounds__(256) void merge_splits_kernel(AttendArgs a, int pad
         lsum += rec[1] * wgt;
         acc += *reinterpret_cast<const floatx4 *>(a.split_scratch + prow(sp) * D + d4 * 4) * wgt;
     }
-    red_o[part][d4] = acc;
-    if (d4 == 0) {
-        red_l[part] = lsum;
-    }
-    __syncthreads();
-    if (part == 0) {
-#pragma unroll
-        for (int k = 1; k < 8; k++) {
-            acc += red_o[k][d4];
-            lsum += red_l[k];
-        }
-        *reinterpret_cast<floatx4 *>(a.out + (int64_t)t * (a.s.h * D) + hh * D + d4 * 4) = acc * (1.f / lsum);
-    }
+    *reinterpret_cast<floatx4 *>(a.out + (int64_t)t * (a.s.h * D) + hh * D + d4 * 4) = acc * (1.f / lsum);
 }
 
 }  // namespace
@@ -540,25 +633,39 @@ hipError_t launch_prefill(const AttendArgs &a, int num_cus, hipStream_t stream) 
     const int rows = heads_per_unit * a.qlen;
     const int n_qtiles = (rows + BM - 1) / BM;
     const int n_items = n_qtiles * units;
-    const int order = (!a.causal || packed) ? 0 : (n_items <= 2 * num_cus ? 2 : 1);
+    // Too few items to give every CU two workgroups: eight-wave workgroups, one per CU (see the kernel).  Measured
+    // on 2048 causal tokens of 32 heads (512 items, 2 to 32 tiles each): 58 us with two four-wave workgroups per
+    // CU, 65 us with one of eight waves (nothing runs beside an item's first tiles and its last stores); on 1024
+    // tokens 29 us against 60 us for four-wave workgroups cut along the keys and merged by a second kernel.
+    const bool two_groups = n_items < 2 * num_cus;
+    const int slots = two_groups ? num_cus : 2 * num_cus;
+    const int order = (!a.causal || packed) ? 0 : (!two_groups && n_items == 2 * num_cus ? 2 : 1);
     // A few tokens against a long cache are a handful of workgroups with hundreds of tiles each: cut the key
-    // range so that the chip is full once, as long as every share keeps at least four tiles and the
-    // partials fit the scratch.
+    // range so that the chip is full once, as long as every share keeps at least four tiles per group of waves
+    // and the partials fit the scratch.
     int nsplit = 1;
-    if (a.split_scratch && n_items < 2 * num_cus) {
+    if (a.split_scratch && n_items < slots) {
         int kv_end = a.kvs;
         const int t_max = packed ? a.qlen : n_qtiles * BM;  // one past the last token of the last tile (or beyond)
         if (a.causal && a.p0 + t_max < kv_end) kv_end = a.p0 + t_max;
         const int n_tiles = (kv_end + BN - 1) / BN;
-        nsplit = (2 * num_cus + n_items - 1) / n_items;
-        if (nsplit > n_tiles / 4) nsplit = n_tiles / 4;
+        const int min_tiles = two_groups ? 8 : 4;
+        nsplit = (slots + n_items - 1) / n_items;
+        if (nsplit > n_tiles / min_tiles) nsplit = n_tiles / min_tiles;
         if (nsplit > kPrefillMaxSplits) nsplit = kPrefillMaxSplits;
         while (nsplit > 1 && (int64_t)nsplit * n_qtiles * BM * units * (D + 2) > a.split_floats) nsplit--;
         if (nsplit < 2) nsplit = 1;
     }
-    hipLaunchKernelGGL(prefill_kernel, dim3(n_items, nsplit), dim3(THREADS), 0, stream, a, n_qtiles, order, packed);
+    if (two_groups) {
+        hipLaunchKernelGGL(prefill_kernel<2>, dim3(n_items, nsplit), dim3(2 * THREADS), 0, stream, a, n_qtiles, order,
+                           packed);
+    } else {
+        hipLaunchKernelGGL(prefill_kernel<1>, dim3(n_items, nsplit), dim3(THREADS), 0, stream, a, n_qtiles, order,
+                           packed);
+    }
     if (nsplit > 1) {
-        hipLaunchKernelGGL(merge_splits_kernel, dim3(rows, units), dim3(256), 0, stream, a, n_qtiles * BM, nsplit, packed);
+        hipLaunchKernelGGL(merge_splits_kernel, dim3((unsigned)(((int64_t)rows * units + 7) / 8)), dim3(256), 0, stream, a,
+                           n_qtiles * BM, nsplit, packed);
     }
     return hipGetLastError();
 }
