@@ -85,30 +85,37 @@ __device__ inline void st_dev4(float *p, uintx4 v) {
 }
 __device__ inline void wait_vm() { asm volatile("s_waitcnt vmcnt(0)" : : : "memory"); }
 
-// Eight 16-byte loads at device scope, all issued before the one wait.  Load i is done by the lanes
+// 1, 2, 4 or 8 16-byte loads at device scope, all issued before the one wait.  Load i is done by the lanes
 // whose bit is set in mask[i]; the other lanes keep what r[i] held.  One block of assembly, so that
 // nothing can touch the destination registers between the loads and the wait.
-__device__ inline void ld_lines8(const float *const (&p)[8], uintx4 (&r)[8], const unsigned long long (&m)[8]) {
+#define GLM_LD_LINE(i) "s_and_b64 exec, %[sv], %[m" #i "]\n\tglobal_load_dwordx4 %[r" #i "], %[p" #i "], off sc1\n\t"
+__device__ inline void ld_lines(const float *const (&p)[1], uintx4 (&r)[1], const unsigned long long (&m)[1]) {
     unsigned long long saved;
-    asm volatile("s_mov_b64 %[sv], exec\n\t"
-                 "s_and_b64 exec, %[sv], %[m0]\n\t"
-                 "global_load_dwordx4 %[r0], %[p0], off sc1\n\t"
-                 "s_and_b64 exec, %[sv], %[m1]\n\t"
-                 "global_load_dwordx4 %[r1], %[p1], off sc1\n\t"
-                 "s_and_b64 exec, %[sv], %[m2]\n\t"
-                 "global_load_dwordx4 %[r2], %[p2], off sc1\n\t"
-                 "s_and_b64 exec, %[sv], %[m3]\n\t"
-                 "global_load_dwordx4 %[r3], %[p3], off sc1\n\t"
-                 "s_and_b64 exec, %[sv], %[m4]\n\t"
-                 "global_load_dwordx4 %[r4], %[p4], off sc1\n\t"
-                 "s_and_b64 exec, %[sv], %[m5]\n\t"
-                 "global_load_dwordx4 %[r5], %[p5], off sc1\n\t"
-                 "s_and_b64 exec, %[sv], %[m6]\n\t"
-                 "global_load_dwordx4 %[r6], %[p6], off sc1\n\t"
-                 "s_and_b64 exec, %[sv], %[m7]\n\t"
-                 "global_load_dwordx4 %[r7], %[p7], off sc1\n\t"
-                 "s_mov_b64 exec, %[sv]\n\t"
-                 "s_waitcnt vmcnt(0)"
+    asm volatile("s_mov_b64 %[sv], exec\n\t" GLM_LD_LINE(0) "s_mov_b64 exec, %[sv]\n\ts_waitcnt vmcnt(0)"
+                 : [sv] "=&s"(saved), [r0] "+v"(r[0])
+                 : [p0] "v"(p[0]), [m0] "s"(m[0])
+                 : "memory", "scc");
+}
+__device__ inline void ld_lines(const float *const (&p)[2], uintx4 (&r)[2], const unsigned long long (&m)[2]) {
+    unsigned long long saved;
+    asm volatile("s_mov_b64 %[sv], exec\n\t" GLM_LD_LINE(0) GLM_LD_LINE(1) "s_mov_b64 exec, %[sv]\n\ts_waitcnt vmcnt(0)"
+                 : [sv] "=&s"(saved), [r0] "+v"(r[0]), [r1] "+v"(r[1])
+                 : [p0] "v"(p[0]), [p1] "v"(p[1]), [m0] "s"(m[0]), [m1] "s"(m[1])
+                 : "memory", "scc");
+}
+__device__ inline void ld_lines(const float *const (&p)[4], uintx4 (&r)[4], const unsigned long long (&m)[4]) {
+    unsigned long long saved;
+    asm volatile("s_mov_b64 %[sv], exec\n\t" GLM_LD_LINE(0) GLM_LD_LINE(1) GLM_LD_LINE(2) GLM_LD_LINE(3)
+                 "s_mov_b64 exec, %[sv]\n\ts_waitcnt vmcnt(0)"
+                 : [sv] "=&s"(saved), [r0] "+v"(r[0]), [r1] "+v"(r[1]), [r2] "+v"(r[2]), [r3] "+v"(r[3])
+                 : [p0] "v"(p[0]), [p1] "v"(p[1]), [p2] "v"(p[2]), [p3] "v"(p[3]), [m0] "s"(m[0]), [m1] "s"(m[1]),
+                   [m2] "s"(m[2]), [m3] "s"(m[3])
+                 : "memory", "scc");
+}
+__device__ inline void ld_lines(const float *const (&p)[8], uintx4 (&r)[8], const unsigned long long (&m)[8]) {
+    unsigned long long saved;
+    asm volatile("s_mov_b64 %[sv], exec\n\t" GLM_LD_LINE(0) GLM_LD_LINE(1) GLM_LD_LINE(2) GLM_LD_LINE(3) GLM_LD_LINE(4)
+                 GLM_LD_LINE(5) GLM_LD_LINE(6) GLM_LD_LINE(7) "s_mov_b64 exec, %[sv]\n\ts_waitcnt vmcnt(0)"
                  : [sv] "=&s"(saved), [r0] "+v"(r[0]), [r1] "+v"(r[1]), [r2] "+v"(r[2]), [r3] "+v"(r[3]),
                    [r4] "+v"(r[4]), [r5] "+v"(r[5]), [r6] "+v"(r[6]), [r7] "+v"(r[7])
                  : [p0] "v"(p[0]), [p1] "v"(p[1]), [p2] "v"(p[2]), [p3] "v"(p[3]), [p4] "v"(p[4]), [p5] "v"(p[5]),
@@ -116,6 +123,7 @@ __device__ inline void ld_lines8(const float *const (&p)[8], uintx4 (&r)[8], con
                    [m4] "s"(m[4]), [m5] "s"(m[5]), [m6] "s"(m[6]), [m7] "s"(m[7])
                  : "memory", "scc");
 }
+#undef GLM_LD_LINE
 
 __device__ inline floatx4 mfma16(half8 a, half8 b, floatx4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
@@ -346,7 +354,7 @@ __device__ inline float reduce_splits(float x, int sl_log, F op) {
     return x;
 }
 
-// Polls lines `first + it * step` (it = 0 .. 7, those below nsplit) of one (quad, piece) until all have
+// Polls lines `first + it * step` (it = 0 .. N - 1, those below nsplit) of one (quad, piece) until all have
 // arrived, then folds them into the lane's (max, sum, O) in the order of their index: the result does not
 // depend on the order in which the lines showed up.  A line counts when all four of its pieces carry the
 // stamp (its log-sum-exp is spread over them).  Returns 1 when the wait ran out.
@@ -354,14 +362,15 @@ struct Fold {
     float m, w;
     floatx4 o;
 };
-__device__ inline int poll_lines(const float *base, int first, int step, int nsplit, bool valid, unsigned int stamp32,
-                                 int piece, unsigned long long t0, unsigned long long limit, Fold &acc) {
-    uintx4 r[8];
-    const float *p[8];
-    bool need[8];
-    unsigned long long pending[8];
+template <int N>
+__device__ inline int poll_lines_n(const float *base, int first, int step, int nsplit, bool valid, unsigned int stamp32,
+                                   int piece, unsigned long long t0, unsigned long long limit, Fold &acc) {
+    uintx4 r[N];
+    const float *p[N];
+    bool need[N];
+    unsigned long long pending[N];
 #pragma unroll
-    for (int it = 0; it < 8; it++) {
+    for (int it = 0; it < N; it++) {
         const int sp = first + it * step;
         r[it] = uintx4{0u, 0u, 0u, 0u};
         need[it] = valid && sp < nsplit;
@@ -371,12 +380,12 @@ __device__ inline int poll_lines(const float *base, int first, int step, int nsp
     TS(13);
     while (true) {
         const unsigned long long now = wall_clock64();  // read while the loads are on their way
-        ld_lines8(p, r, pending);                       // only what has not arrived yet is loaded again
+        ld_lines(p, r, pending);                        // only what has not arrived yet is loaded again
         TSCOUNT(14);
         TS(15);
         unsigned long long any = 0ull;
 #pragma unroll
-        for (int it = 0; it < 8; it++) {
+        for (int it = 0; it < N; it++) {
             if (pending[it] != 0ull) {
                 // all four pieces of a line: and over the quad of lanes
                 int ok = !need[it] || r[it][0] == stamp32;
@@ -396,10 +405,10 @@ __device__ inline int poll_lines(const float *base, int first, int step, int nsp
     }
     TS(12);
     // the base-2 log-sum-exp of each line from the bytes in its four pieces, and the new max
-    float lse[8];
+    float lse[N];
     float m_new = acc.m;
 #pragma unroll
-    for (int it = 0; it < 8; it++) {
+    for (int it = 0; it < N; it++) {
         int bits = (int)(r[it][3] >> 24) << (8 * piece);
         bits |= __builtin_amdgcn_update_dpp(0, bits, 0xB1, 0xf, 0xf, true);
         bits |= __builtin_amdgcn_update_dpp(0, bits, 0x4E, 0xf, 0xf, true);
@@ -412,7 +421,7 @@ __device__ inline int poll_lines(const float *base, int first, int step, int nsp
         acc.o *= sc;
         acc.m = m_new;
 #pragma unroll
-        for (int it = 0; it < 8; it++) {
+        for (int it = 0; it < N; it++) {
             const float wgt = __builtin_amdgcn_exp2f(lse[it] - m_new);  // 0 for lines that are not there
             const floatx4 v = unpack_piece(r[it]);
             acc.w += wgt;
@@ -423,6 +432,19 @@ __device__ inline int poll_lines(const float *base, int first, int step, int nsp
         }
     }
     return 0;
+}
+
+// b0: the first split of the pass (first = b0 + the lane's split slot).  The code that runs is the one for the
+// number of lines the pass really has per lane: at 2.3 ns a vector instruction, folding lines that are not
+// there costs as much as folding lines that are.
+__device__ inline int poll_lines(const float *base, int b0, int first, int step, int nsplit, bool valid,
+                                 unsigned int stamp32, int piece, unsigned long long t0, unsigned long long limit,
+                                 Fold &acc) {
+    const int n = (nsplit - b0 + step - 1) / step;  // the same in every lane
+    if (n <= 1) return poll_lines_n<1>(base, first, step, nsplit, valid, stamp32, piece, t0, limit, acc);
+    if (n <= 2) return poll_lines_n<2>(base, first, step, nsplit, valid, stamp32, piece, t0, limit, acc);
+    if (n <= 4) return poll_lines_n<4>(base, first, step, nsplit, valid, stamp32, piece, t0, limit, acc);
+    return poll_lines_n<8>(base, first, step, nsplit, valid, stamp32, piece, t0, limit, acc);
 }
 
 // What ends a slice: the (max, sum, O) of all lanes of a piece merged, normalised and stored.
@@ -456,7 +478,7 @@ __device__ inline int merge_quads(const MergeGeom &mg, int q_begin, int q_end, i
         const float *base = mg.part_g + ((int64_t)(hd * QUADS + quad) * mg.nsplit * 4 + piece) * 4;
         Fold acc = {-INFINITY, 0.f, floatx4{0.f, 0.f, 0.f, 0.f}};
         for (int b0 = 0; b0 < mg.nsplit; b0 += 8 * SL) {
-            if (poll_lines(base, b0 + s, SL, mg.nsplit, valid, mg.stamp32, piece, t0, limit, acc)) {
+            if (poll_lines(base, b0, b0 + s, SL, mg.nsplit, valid, mg.stamp32, piece, t0, limit, acc)) {
                 return 1;
             }
         }
@@ -491,6 +513,7 @@ struct DecodeShared {
     float pnew[16];     // probability of the new token
     __attribute__((aligned(16))) __half knew[D];  // its key, roped, fp16
     __attribute__((aligned(16))) __half q[16][QPAD];  // the group's queries, roped, scaled, fp16
+    int k_issued;       // score waves whose first tile loads are in the memory pipeline
     int q_ready;        // score waves that have left their part of the queries
     int m_ready;        // score waves that have left their maxes, over all rounds
     int p_ready;        // score waves that have left their part of P, over all rounds
@@ -545,7 +568,7 @@ __device__ inline int merge_quad4(const MergeGeom &mg, DecodeShared &sh, int q, 
     Fold acc = {-INFINITY, 0.f, floatx4{0.f, 0.f, 0.f, 0.f}};
     int failed = 0;
     for (int b0 = 0; b0 < mg.nsplit && !failed; b0 += 8 * 64) {
-        failed = poll_lines(base, b0 + s, 64, mg.nsplit, true, mg.stamp32, piece, t0, limit, acc);
+        failed = poll_lines(base, b0, b0 + s, 64, mg.nsplit, true, mg.stamp32, piece, t0, limit, acc);
     }
     reduce_fold(acc, 4);
     TS(4);
@@ -612,7 +635,15 @@ struct Geom {
     int tb, te, rounds;
     bool owner_wg;
     unsigned long long t_start;
+    unsigned long long gen_v;  // the launch count as loaded, in vector registers (see decode_body)
 };
+
+// A use of v that costs nothing: the load that produces v cannot be moved below this point, and the wave
+// waits here for that load (and for no later one).
+__device__ inline void pin_value(unsigned long long v) {
+    const unsigned int lo = (unsigned int)v, hi = (unsigned int)(v >> 32);
+    asm volatile("" : : "v"(lo), "v"(hi));
+}
 
 // ---- score waves: S^T = K q^T of one tile per round, the softmax across the workgroup's tiles, P to LDS
 template <int TYPE>
@@ -632,7 +663,8 @@ __device__ inline void score_wave(const DecodeArgs &a, DecodeShared &sh, const G
         pos[1] = clamp_position(pos[1], a.rope.table_positions, a.flags);
     }
     // loads of a wave return in order: the small rows first, so that the queries can be prepared while
-    // the K tile is on its way
+    // the K tile is on its way.  (Left to the output waves, the queries come late: their loads queue up
+    // behind the score waves' tiles in the CU's memory pipeline.)
     QPart qpart;
     const int q_hd = 4 * w + (lane >> 4), q_d0 = (lane & 15) * 8;
     {
@@ -646,8 +678,12 @@ __device__ inline void score_wave(const DecodeArgs &a, DecodeShared &sh, const G
     int nk = ge.te - ge.tb < W ? ge.te - ge.tb : W;
     half8 kf[4][4];
     load_k_tile(Kg, L, (ge.tb + (w < nk ? w : 0)) * TILE, lane, kf);
+    if (lane == 0) {
+        __hip_atomic_fetch_add(&sh.k_issued, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
     TS(0);
     *reinterpret_cast<half8 *>(&sh.q[q_hd][q_d0]) = finish_q_part<TYPE>(qpart, q_d0, a.scale, q_hd >= G);
+    pin_value(ge.gen_v);  // older than the query loads that have just been waited for
     lds_signal(&sh.q_ready, lane);
     lds_wait_ge(&sh.q_ready, W, a.flags);
     half8 qf[4];
@@ -776,6 +812,9 @@ __device__ inline void output_wave(const DecodeArgs &a, DecodeShared &sh, const 
 
     int nk = ge.te - ge.tb < W ? ge.te - ge.tb : W;
     half8 vf[2][8];
+    // The K tiles go into the CU's memory pipeline first: the scores, the maxes and the probabilities are
+    // all made from them while the V columns, which only the last step needs, are still on their way.
+    lds_wait_ge(&sh.k_issued, W, a.flags);
     load_v_dims<0, 8>(Vg, L, ge.tb * TILE, nk, w, lane, vf);
     float vnew[2][4];
     if (ge.owner_wg) {
@@ -798,6 +837,7 @@ __device__ inline void output_wave(const DecodeArgs &a, DecodeShared &sh, const 
         }
     }
     TS(0);
+    pin_value(ge.gen_v);  // nothing to do before P anyway
     o[0] = floatx4{0.f, 0.f, 0.f, 0.f};
     o[1] = floatx4{0.f, 0.f, 0.f, 0.f};
     float m_run = -INFINITY;
@@ -896,9 +936,20 @@ __device__ inline void decode_body(const DecodeArgs &a, DecodeShared &sh) {
     ge.owner_wg = split == a.nsplit - 1;  // appends the new token and attends to it
 
     // The launch count stamps this launch's lines.  Every lane reads it (no branch, one request per
-    // wave) among its first loads: no workgroup can have finished before that.
-    const unsigned long long gen = __hip_atomic_load(&a.sync[g].gen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    const unsigned int stamp32 = a.stamp_groups ? decode_stamp_grouped(gen, g) : decode_stamp(gen);
+    // wave) as its first load: no workgroup can have finished before that.  The load goes to the memory
+    // side and takes about a microsecond: its value stays in vector registers, behind an address the
+    // compiler cannot prove uniform, until the wave's tile loads have been issued and used (`resolve`),
+    // or the wave would sit out that microsecond before it asks for its first tile.
+    const unsigned long long *gen_at = &a.sync[g].gen;
+    asm volatile("" : "+v"(gen_at));
+    // (address space 1: a global load; a flat one would also stand in the way of every wait for LDS)
+    const unsigned long long gen_v =
+        __hip_atomic_load(reinterpret_cast<const __attribute__((address_space(1))) unsigned long long *>(
+                              reinterpret_cast<uintptr_t>(gen_at)),
+                          __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    ge.gen_v = gen_v;
+    unsigned long long gen = 0ull, stamp = 0ull;
+    unsigned int stamp32 = 0u;
 
     const int total_quads = G * QUADS;
     const int qps = (total_quads + a.nsplit - 1) / a.nsplit;  // quads per slice
@@ -909,20 +960,30 @@ __device__ inline void decode_body(const DecodeArgs &a, DecodeShared &sh) {
     while (mg.sl_log < 4 && (1 << mg.sl_log) < a.nsplit) {
         mg.sl_log++;
     }
-    mg.stamp32 = stamp32;
+    // ... but no more split lanes than leave a wave room for its share of the slice's quads in one pass
+    while (mg.sl_log > 0 && (16 >> mg.sl_log) * W < qps) {
+        mg.sl_log--;
+    }
     mg.part_g = a.part + (int64_t)g * a.nsplit * kDecodePartFloats;
     mg.out_g = a.out + (int64_t)g * G * D;
     mg.gen_word = &a.sync[g].gen;
-    mg.gen_next = decode_next_gen(gen);
     DecodeGroupSync *sy = a.sync + g;
     unsigned long long *claim = a.claim + (int64_t)g * kDecodeMaxSplits;
-    const unsigned long long stamp = gen + 1ull;
+    auto resolve = [&]() {
+        gen = ((unsigned long long)__builtin_amdgcn_readfirstlane((unsigned int)(gen_v >> 32)) << 32) |
+              (unsigned long long)__builtin_amdgcn_readfirstlane((unsigned int)gen_v);
+        stamp32 = a.stamp_groups ? decode_stamp_grouped(gen, g) : decode_stamp(gen);
+        stamp = gen + 1ull;
+        mg.stamp32 = stamp32;
+        mg.gen_next = decode_next_gen(gen);
+    };
 
     if (scores) {
         score_wave<TYPE>(a, sh, ge);
         if (a.nsplit == 1) {
             return;
         }
+        resolve();
 #ifdef EXP_NO_MERGE
         return;
 #endif
@@ -979,6 +1040,7 @@ __device__ inline void decode_body(const DecodeArgs &a, DecodeShared &sh) {
     floatx4 o[2];
     float l_tot, m_fin;
     output_wave(a, sh, ge, o, l_tot, m_fin);
+    resolve();
     if (a.nsplit == 1) {
         // a single workgroup saw every key of the group: normalise and finish
         if (j < G) {
@@ -1046,6 +1108,7 @@ __device__ inline void decode_body(const DecodeArgs &a, DecodeShared &sh) {
 __global__ __launch_bounds__(kBlock) void decode_kernel(DecodeArgs a) {
     __shared__ DecodeShared sh;
     if (threadIdx.x == 0) {
+        sh.k_issued = 0;
         sh.q_ready = 0;
         sh.m_ready = 0;
         sh.p_ready = 0;

@@ -286,6 +286,9 @@ int do_decode(glm_attn_ctx *c, int layer, const float *qkv, const int32_t *posit
     if (nsplit > cu_share) nsplit = cu_share;
     if (nsplit > c->max_splits) nsplit = c->max_splits;
     if (shared && nsplit > kStaticMaxParts / c->shape.kvh) nsplit = kStaticMaxParts / c->shape.kvh;
+    // One round of tiles is over sooner in one workgroup than the exchange between several takes (a second
+    // round in the same workgroup is not: it costs 3 us, the exchange 2).
+    if (n_tiles <= kDecodeMaxWaves) nsplit = 1;
     da.nsplit = nsplit;
     da.tiles_q = n_tiles / nsplit;
     da.tiles_r = n_tiles % nsplit;
