@@ -652,6 +652,7 @@ __device__ inline void score_wave(const DecodeArgs &a, DecodeShared &sh, const G
     const int L = a.s.L, G = a.s.G;
     const __half *Kg = a.k_cache + (int64_t)g * L * D;
     const bool owner = ge.owner_wg && w == W - 1;
+    TS(5);
 
     int pos[2] = {a.pos0, a.pos1};
     if (TYPE != GLM_ATTN_ROPE_DISABLED) {
@@ -677,6 +678,7 @@ __device__ inline void score_wave(const DecodeArgs &a, DecodeShared &sh, const G
     }
     int nk = ge.te - ge.tb < W ? ge.te - ge.tb : W;
     half8 kf[4][4];
+    TS(8);
     load_k_tile(Kg, L, (ge.tb + (w < nk ? w : 0)) * TILE, lane, kf);
     if (lane == 0) {
         __hip_atomic_fetch_add(&sh.k_issued, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
@@ -951,25 +953,30 @@ __device__ inline void decode_body(const DecodeArgs &a, DecodeShared &sh) {
     unsigned long long gen = 0ull, stamp = 0ull;
     unsigned int stamp32 = 0u;
 
+    // What the exchange needs is worked out after the wave's own part (`resolve`): ahead of it, it would
+    // stand between the start of the wave and its first loads.
     const int total_quads = G * QUADS;
-    const int qps = (total_quads + a.nsplit - 1) / a.nsplit;  // quads per slice
+    int qps = 0;  // quads per slice
     MergeGeom mg;
-    mg.nsplit = a.nsplit;
-    mg.G = G;
-    mg.sl_log = 0;
-    while (mg.sl_log < 4 && (1 << mg.sl_log) < a.nsplit) {
-        mg.sl_log++;
-    }
-    // ... but no more split lanes than leave a wave room for its share of the slice's quads in one pass
-    while (mg.sl_log > 0 && (16 >> mg.sl_log) * W < qps) {
-        mg.sl_log--;
-    }
-    mg.part_g = a.part + (int64_t)g * a.nsplit * kDecodePartFloats;
-    mg.out_g = a.out + (int64_t)g * G * D;
-    mg.gen_word = &a.sync[g].gen;
-    DecodeGroupSync *sy = a.sync + g;
-    unsigned long long *claim = a.claim + (int64_t)g * kDecodeMaxSplits;
+    DecodeGroupSync *sy = nullptr;
+    unsigned long long *claim = nullptr;
     auto resolve = [&]() {
+        qps = (total_quads + a.nsplit - 1) / a.nsplit;
+        mg.nsplit = a.nsplit;
+        mg.G = G;
+        mg.sl_log = 0;
+        while (mg.sl_log < 4 && (1 << mg.sl_log) < a.nsplit) {
+            mg.sl_log++;
+        }
+        // ... but no more split lanes than leave a wave room for its share of the slice's quads in one pass
+        while (mg.sl_log > 0 && (16 >> mg.sl_log) * W < qps) {
+            mg.sl_log--;
+        }
+        mg.part_g = a.part + (int64_t)g * a.nsplit * kDecodePartFloats;
+        mg.out_g = a.out + (int64_t)g * G * D;
+        mg.gen_word = &a.sync[g].gen;
+        sy = a.sync + g;
+        claim = a.claim + (int64_t)g * kDecodeMaxSplits;
         gen = ((unsigned long long)__builtin_amdgcn_readfirstlane((unsigned int)(gen_v >> 32)) << 32) |
               (unsigned long long)__builtin_amdgcn_readfirstlane((unsigned int)gen_v);
         stamp32 = a.stamp_groups ? decode_stamp_grouped(gen, g) : decode_stamp(gen);
