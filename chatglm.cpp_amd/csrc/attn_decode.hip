@@ -814,6 +814,14 @@ __device__ inline void output_wave(const DecodeArgs &a, DecodeShared &sh, const 
 
     int nk = ge.te - ge.tb < W ? ge.te - ge.tb : W;
     half8 vf[2][8];
+    // the new token's v, in the workgroup that appends it: asked for ahead of the V columns (loads of a
+    // wave return in order, and two small loads behind them would be waited for one after the other)
+    floatx4 vraw_new[2] = {floatx4{0.f, 0.f, 0.f, 0.f}, floatx4{0.f, 0.f, 0.f, 0.f}};
+    if (ge.owner_wg) {
+        const float *vhead = a.qkv + a.lay.v_off + (int64_t)g * a.lay.head_stride + w * 32;
+        vraw_new[0] = *reinterpret_cast<const floatx4 *>(vhead + c * 4);
+        vraw_new[1] = *reinterpret_cast<const floatx4 *>(vhead + 16 + c * 4);
+    }
     // The K tiles go into the CU's memory pipeline first: the scores, the maxes and the probabilities are
     // all made from them while the V columns, which only the last step needs, are still on their way.
     lds_wait_ge(&sh.k_issued, W, a.flags);
@@ -821,10 +829,9 @@ __device__ inline void output_wave(const DecodeArgs &a, DecodeShared &sh, const 
     float vnew[2][4];
     if (ge.owner_wg) {
         // chatglm.cpp:672-675: v of the new token goes to the cache as fp16, and into this launch's output
-        const float *vhead = a.qkv + a.lay.v_off + (int64_t)g * a.lay.head_stride + w * 32;
 #pragma unroll
         for (int jb = 0; jb < 2; jb++) {
-            const floatx4 vraw = *reinterpret_cast<const floatx4 *>(vhead + jb * 16 + c * 4);
+            const floatx4 vraw = vraw_new[jb];
             _Float16 v16[4];
 #pragma unroll
             for (int e = 0; e < 4; e++) {
@@ -932,10 +939,14 @@ __device__ inline void decode_body(const DecodeArgs &a, DecodeShared &sh) {
     const int lane = ge.lane, w = ge.w, j = ge.j, c = ge.c, g = ge.g, split = ge.split;
     const int G = a.s.G;
     // tiles [tb, te) of the keys already in the cache are this workgroup's
-    ge.tb = split * a.tiles_q + (split < a.tiles_r ? split : a.tiles_r);
-    ge.te = ge.tb + a.tiles_q + (split < a.tiles_r ? 1 : 0);
+    // (the last tiles_r splits take one tile more)
+    const int extra_from = a.nsplit - a.tiles_r;
+    ge.tb = split * a.tiles_q + (split > extra_from ? split - extra_from : 0);
+    ge.te = ge.tb + a.tiles_q + (split >= extra_from ? 1 : 0);
     ge.rounds = ge.te - ge.tb > W ? (ge.te - ge.tb + W - 1) / W : 1;
-    ge.owner_wg = split == a.nsplit - 1;  // appends the new token and attends to it
+    // The first workgroup also appends the new token and attends to it: every merge waits for its lines,
+    // so it is the one that is dispatched first and never has the extra tile.
+    ge.owner_wg = split == 0;
 
     // The launch count stamps this launch's lines.  Every lane reads it (no branch, one request per
     // wave) as its first load: no workgroup can have finished before that.  The load goes to the memory
