@@ -103,6 +103,52 @@ def read_ceilings(torch, pkg, kv, layer_halfs, stream, warmup, steps):
     return out
 
 
+def timelines(torch, pkg, capi):
+    """In-kernel clock readings of the instrumented build: the decode launch of the headline workload and causal
+    prompts of the ChatGLM3-6B shape.  Times are us since the first wave of the launch started; reading the clock
+    costs about 0.1 us a time, so the instrumented kernels run a little longer than the plain ones."""
+    import numpy as np
+
+    dev = torch.device("cuda:0")
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(99)
+    out = {}
+    slot = np.arange(capi.TIMELINE_SLOTS)
+    # decode, GLM-4-9B shape at 32k: 4 layers' caches, the last launch's readings
+    layers = 4
+    ctx = pkg.Context(num_layers=layers, num_attention_heads=H, num_key_value_heads=KVH, head_size=D,
+                      max_length=MAX_LENGTH, max_qlen=1)
+    width = (H + 2 * KVH) * D
+    qkv = torch.randn(layers, width, generator=gen, device=dev, dtype=torch.float32)
+    o = torch.zeros(layers, H * D, device=dev, dtype=torch.float32)
+    for n_past in (N_PAST_DECODE, 4095):
+        for _ in range(3):
+            for l in range(layers):
+                pkg.check(ctx.forward(l, qkv[l].data_ptr(), 1, n_past, o[l].data_ptr(), position_ids_host=[n_past]),
+                          "glm_attn_forward")
+        torch.cuda.synchronize()
+        t = capi.read_timeline("decode")
+        out[f"decode_kernel, n_past {n_past}"] = {
+            "score waves": capi.summarise_timeline(t, capi.DECODE_STAMPS["score"], (slot % 8) < 4),
+            "output waves": capi.summarise_timeline(t, capi.DECODE_STAMPS["output"], (slot % 8) >= 4)}
+    ctx.close()
+    # causal prompts at n_past 0, ChatGLM3-6B shape (32 heads, 2 KV groups, max_length 8192)
+    ctx = pkg.Context(num_layers=1, num_attention_heads=32, num_key_value_heads=2, head_size=128, max_length=8192,
+                      max_qlen=2048)
+    for qlen in (2048, 512):
+        qkv = torch.randn(qlen, width, generator=gen, device=dev, dtype=torch.float32)
+        o = torch.zeros(qlen, 32 * 128, device=dev, dtype=torch.float32)
+        pos = torch.arange(qlen, device=dev, dtype=torch.int32)
+        for _ in range(3):
+            pkg.check(ctx.forward(0, qkv.data_ptr(), qlen, 0, o.data_ptr(), position_ids_ptr=pos.data_ptr()),
+                      "glm_attn_forward")
+        torch.cuda.synchronize()
+        t = capi.read_timeline("prefill")
+        out[f"prefill_kernel, {qlen} causal tokens"] = capi.summarise_timeline(t, capi.PREFILL_STAMPS, slot >= 0)
+    ctx.close()
+    return out
+
+
 class optional_section:
     """The sections beyond the contract's line (projections, whole layers, whole model) must not take the line with
     them: an exception inside one is recorded as that section's "error" and the run goes on."""
@@ -141,6 +187,9 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB device copy (known size) so that FETCH_SIZE / WRITE_SIZE "
                          "counters of a profiled run can be scaled")
+    ap.add_argument("--timeline", action="store_true",
+                    help="not a timing run: load the instrumented library (libglm_attn_timeline.so), run the decode "
+                         "step and a causal prompt once and print where the waves' time went (in-kernel clock)")
     args = ap.parse_args()
     if args.ceiling_only:
         args.ceiling = True
@@ -155,8 +204,15 @@ def main():
     from __graft_entry__ import load_package
 
     pkg = load_package()
+    if args.timeline:
+        import chatglm_cpp_amd.capi as capi
+
+        capi.use_timeline_build()
     pkg.lib()  # fails loudly if libglm_attn.so is missing
     assert torch.cuda.is_available(), "bench.py needs a GPU"
+    if args.timeline:
+        print(json.dumps({"timeline": timelines(torch, pkg, capi)}))
+        return
     dev = torch.device("cuda:0")
     torch.cuda.set_device(0)
 

@@ -140,6 +140,71 @@ def build(verbose=False):
 
 _lib = None
 
+# The instrumented build (csrc/Makefile, target `timeline`): the same library whose decode and prefill kernels
+# leave clock readings per wave.  For finding where the time of a launch goes, never for timing it.
+TIMELINE_LIB_PATH = os.path.join(_PKG, "libglm_attn_timeline.so")
+TIMELINE_SLOTS = 4096  # waves recorded (kTimelineSlots)
+# index -> what the wave had just done when it read the clock; slot = workgroup * 8 + wave, waves 0-3 of a
+# decode workgroup are score waves, 4-7 output waves
+DECODE_STAMPS = {
+    "score": [(10, "wave started"), (5, "own work entered"), (8, "query loads issued"), (0, "K tile loads issued"),
+              (1, "queries in LDS (and the new key)"), (2, "maxes of the last round left"),
+              (3, "probabilities of the last round left"), (6, "first look at the others' lines"),
+              (13, "polling entered (last pass)"), (15, "last poll's loads back"), (12, "all lines in (last pass)"),
+              (4, "folded within the wave"), (11, "slice folded"), (7, "slice written")],
+    "output": [(10, "wave started"), (0, "V column loads issued"), (3, "probabilities seen"), (4, "second product done"),
+               (5, "lines issued")],
+}
+PREFILL_STAMPS = [(0, "wave started"), (1, "first copies issued"), (2, "first tiles landed"), (3, "first product done"),
+                  (8, "1st tile of the group done"), (9, "2nd tile done"), (10, "4th tile done"), (4, "tile loop done"),
+                  (5, "last second product done"), (6, "the two groups merged"), (7, "output stores issued")]
+
+
+def use_timeline_build():
+    """Makes lib() load the instrumented library.  Call before anything else of this module."""
+    global LIB_PATH
+    if _lib is not None:
+        raise RuntimeError("the library is already loaded")
+    LIB_PATH = TIMELINE_LIB_PATH
+
+
+def read_timeline(kind):
+    """Clock readings (100 MHz ticks) of the launches since the last call: array [TIMELINE_SLOTS][16] of int64, zero
+    where a wave left none.  kind: "decode" or "prefill".  Only with the instrumented library."""
+    import numpy as np
+
+    fn = getattr(lib(), f"glm_attn_debug_{kind}_timeline", None)
+    if fn is None:
+        raise RuntimeError("timeline readings need the instrumented library: call use_timeline_build() first")
+    fn.argtypes = [ctypes.c_void_p, ctypes.c_size_t]
+    fn.restype = ctypes.c_int
+    n = TIMELINE_SLOTS * 16
+    buf = (ctypes.c_ulonglong * n)()
+    rc = fn(buf, n)
+    if rc != 0:
+        raise RuntimeError(f"glm_attn_debug_{kind}_timeline: hip error {rc}")
+    return np.frombuffer(buf, dtype=np.uint64).reshape(TIMELINE_SLOTS, 16).astype(np.int64)
+
+
+def summarise_timeline(t, stamps, rows):
+    """Per stamp: waves that left one, and min / mean / max in us since the first wave of the launch started.
+    rows: boolean mask over the slots (e.g. the score waves)."""
+    start_idx = stamps[0][0]
+    used = (t[:, start_idx] > 0) & rows
+    if not used.any():
+        return []
+    t0 = t[(t[:, start_idx] > 0), start_idx].min()
+    out = []
+    for idx, name in stamps:
+        v = t[used, idx]
+        v = v[v >= t0]
+        if v.size == 0:
+            continue
+        us = (v - t0) / 100.0
+        out.append({"stamp": name, "waves": int(v.size), "min_us": round(float(us.min()), 2),
+                    "mean_us": round(float(us.mean()), 2), "max_us": round(float(us.max()), 2)})
+    return out
+
 
 def lib():
     global _lib

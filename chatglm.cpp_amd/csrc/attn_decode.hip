@@ -2,27 +2,30 @@
 //
 // One launch does rope(q, k), the K/V append and the attention of one layer (chatglm.cpp:655-717 for
 // qlen == 1).  The cache sequence of each KV group is cut into 64-key tiles that are dealt out to
-// nsplit workgroups x 4 wavefronts.  A wave is on its own until its tiles are done: it issues the
-// few loads of the group's query rows first, then the 32 loads of a whole tile (16 KiB of K rows and
-// 16 KiB of V columns, streaming loads), and ropes, scales and rounds the queries in registers while
-// the tile is in flight; nothing goes through LDS and no wave waits for another one.  The up to 16
-// query heads of the group are the 16 columns of v_mfma_f32_16x16x32_f16 tiles: S^T = K q^T puts keys
-// on the rows, which is exactly the layout the second product O^T = V^T P^T wants for P^T, so
-// probabilities go from accumulator registers to operand registers without touching LDS.
+// nsplit workgroups, up to four tiles (256 keys) a round.  A workgroup is eight waves with two kinds of
+// work: score wave w loads the K rows of tile w, prepares a quarter of the group's queries while they
+// are on their way (rope, scale, fp16), computes S^T = K q^T for all heads of the group and, with the
+// other score waves, the round's softmax, and leaves P in LDS; output wave w loads the V columns of 32
+// output dims for all keys of the round and accumulates O^T = V^T P^T for those dims.  The up to 16
+// query heads of the group are the 16 columns of v_mfma_f32_16x16x32_f16 tiles.  Waves hand over through
+// counters in LDS (no workgroup barrier after the first), and O never leaves the registers of the
+// output waves.
 //
-// The four waves of a workgroup merge their (max, sum, O) through LDS.  Across workgroups the merge
-// happens in the same launch: every workgroup leaves its partial in memory as self-validating 64-byte
-// lines, one per (head, 16 output dims), and one wave of every workgroup then folds the lines of all
-// splits for one such slice of the output.
+// Across workgroups the merge happens in the same launch: every workgroup leaves its partial in memory
+// as self-validating 64-byte lines, one per (head, 16 output dims), stamped with the launch count, and
+// the score waves of every workgroup then fold the lines of all splits for one slice of the output,
+// polling them past the caches until they carry this launch's stamp.  The wait is bounded, and a slice
+// whose wait ran out is redone by a later workgroup (decode_body).
 //
-// The new token's K and V never take part in a cache load of this launch: one wave of each group
-// ropes them, stores them to the cache and starts its softmax state from them, all in registers.
+// The new token's K and V never take part in a cache load of this launch: the first workgroup of each
+// group ropes and appends them and attends to them from registers.
 #include "glm_attn_internal.h"
 
 namespace glm_attn {
 
 #ifdef GLM_ATTN_TIMELINE
-// Instrumented build (csrc/Makefile, target `timeline`): every wave leaves 100 MHz clock readings here.
+// Instrumented build (csrc/Makefile, target `timeline`): every wave leaves 100 MHz clock readings here,
+// 16 per wave; DecodeTimelineStamp in glm_attn_internal.h names them.
 __device__ unsigned long long g_decode_timeline[kTimelineSlots * 16];
 #define TS(i)                                                                                                \
     do {                                                                                                     \
@@ -496,12 +499,10 @@ __device__ inline int merge_quads(const MergeGeom &mg, int q_begin, int q_end, i
     return 0;
 }
 
-#ifndef EXP_DELAY_DIV
-#define EXP_DELAY_DIV 8
-#endif
-#ifndef EXP_DELAY_ADD
-#define EXP_DELAY_ADD 30
-#endif
+// Before its first look at the lines of the others a wave waits an eighth of its own run time so far plus
+// 0.3 us (see decode_body).
+constexpr int kFirstLookDiv = 8;
+constexpr int kFirstLookTicks = 30;  // of the 100 MHz clock
 constexpr int PPITCH = W * TILE + 8;  // row pitch of the P tile in LDS (halfs): conflict-free 16-byte accesses
 constexpr int kBlock = 2 * W * 64;    // W score waves, then W output waves
 
@@ -1002,9 +1003,6 @@ __device__ inline void decode_body(const DecodeArgs &a, DecodeShared &sh) {
             return;
         }
         resolve();
-#ifdef EXP_NO_MERGE
-        return;
-#endif
         // ---- grid-wide merge.  The score waves of every workgroup fold the quads of one slice of the
         // group's output from the lines of all splits, which they load past the caches and poll until
         // they carry this launch's stamp.  The poll is bounded: a wave whose wait runs out flags the
@@ -1027,7 +1025,7 @@ __device__ inline void decode_body(const DecodeArgs &a, DecodeShared &sh) {
         // time later, and a line takes a while to become visible: looking right away would load nearly
         // every line twice, so the first look waits a little.
         {
-            const unsigned long long wait_ticks = (t0 - ge.t_start) / EXP_DELAY_DIV + EXP_DELAY_ADD;
+            const unsigned long long wait_ticks = (t0 - ge.t_start) / kFirstLookDiv + kFirstLookTicks;
             while (wall_clock64() - t0 < wait_ticks && wait_ticks < limit) {
                 __builtin_amdgcn_s_sleep(4);
             }
@@ -1088,9 +1086,6 @@ __device__ inline void decode_body(const DecodeArgs &a, DecodeShared &sh) {
         }
     }
     TS(5);
-#ifdef EXP_NO_TICKET
-    return;
-#endif
     // ---- once the lines of the whole workgroup have been performed: has anybody left a slice behind?
     wait_vm();  // this wave's line stores have been performed
     lds_signal(&sh.stored, lane);
@@ -1158,10 +1153,15 @@ __global__ __launch_bounds__(kBlock) void decode_kernel(DecodeArgs a) {
 }  // namespace
 
 #ifdef GLM_ATTN_TIMELINE
-// Only in the instrumented build: copies the clock readings of the last decode launch to the host.
+// Only in the instrumented build: copies the clock readings of the decode launches since the last call to the
+// host (a later launch overwrites an earlier one's; the count at index 14 adds up) and clears them.
 extern "C" int glm_attn_debug_decode_timeline(unsigned long long *host, size_t n) {
     if (n > (size_t)kTimelineSlots * 16) n = (size_t)kTimelineSlots * 16;
-    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(g_decode_timeline), n * sizeof(unsigned long long));
+    hipError_t e = hipMemcpyFromSymbol(host, HIP_SYMBOL(g_decode_timeline), n * sizeof(unsigned long long));
+    void *at = nullptr;
+    if (e == hipSuccess) e = hipGetSymbolAddress(&at, HIP_SYMBOL(g_decode_timeline));
+    if (e == hipSuccess) e = hipMemset(at, 0, sizeof(unsigned long long) * kTimelineSlots * 16);
+    return (int)e;
 }
 #endif
 

@@ -15,16 +15,25 @@
 namespace glm_attn {
 
 #ifdef GLM_ATTN_TIMELINE
-// Instrumented build: every wave of prefill_kernel leaves 100 MHz clock readings here.
+// Instrumented build (csrc/Makefile, target `timeline`): every wave of prefill_kernel leaves 100 MHz clock
+// readings here, 16 per wave: 0 start, 1 first copies issued, 2 first tiles landed, 3 first product done,
+// 8 / 9 / 10 end of the group's 1st / 2nd / 4th tile, 4 end of the tile loop, 5 last second product done,
+// 6 the two groups merged, 7 output stores issued.
 __device__ unsigned long long g_prefill_timeline[kTimelineSlots * 16];
 #define PTS(i)                                                                                                   \
     do {                                                                                                         \
         const int slot_ = (blockIdx.y * gridDim.x + blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6);        \
         if ((threadIdx.x & 63) == 0 && slot_ < kTimelineSlots) g_prefill_timeline[slot_ * 16 + (i)] = wall_clock64(); \
     } while (0)
+// copies the readings of the launches since the last call to the host (a later launch overwrites an earlier
+// one's) and clears them
 extern "C" int glm_attn_debug_prefill_timeline(unsigned long long *host, size_t n) {
     if (n > (size_t)kTimelineSlots * 16) n = (size_t)kTimelineSlots * 16;
-    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(g_prefill_timeline), n * sizeof(unsigned long long));
+    hipError_t e = hipMemcpyFromSymbol(host, HIP_SYMBOL(g_prefill_timeline), n * sizeof(unsigned long long));
+    void *at = nullptr;
+    if (e == hipSuccess) e = hipGetSymbolAddress(&at, HIP_SYMBOL(g_prefill_timeline));
+    if (e == hipSuccess) e = hipMemset(at, 0, sizeof(unsigned long long) * kTimelineSlots * 16);
+    return (int)e;
 }
 #else
 #define PTS(i) \
