@@ -103,6 +103,48 @@ def read_ceilings(torch, pkg, kv, layer_halfs, stream, warmup, steps):
     return out
 
 
+def mfma_ceilings(torch, pkg, stream):
+    """Loops of matrix instructions (two waves per SIMD on every CU, operands with random bits), each long enough for
+    the clock to settle: what the matrix pipes give any kernel here, beside the prefill kernel's rate."""
+    import ctypes
+
+    lib = pkg.lib()
+    dev = torch.device("cuda:0")
+    operands = (torch.rand(1 << 16, device=dev, dtype=torch.float32) - 0.5).to(torch.float16)  # 128 KiB
+    sink = torch.zeros(1, dtype=torch.float32, device=dev)
+    sh = stream.cuda_stream
+    out = {"workload": "2 workgroups of 4 waves per CU; per wave 2000 iterations of 32 32x32x16 (64 16x16x32) matrix "
+                       "instructions; the 'mix' forms add one 16-byte-per-lane LDS read per 32x32x16 and 21 vector "
+                       "instructions (4 v_exp_f32) per four, the prefill kernel's diet"}
+    for name, pattern in (("mfma_32x32x16_f16", pkg.BENCH_MFMA_32X32X16), ("mfma_16x16x32_f16", pkg.BENCH_MFMA_16X16X32),
+                          ("mfma_32x32x16_f16_mix", pkg.BENCH_MFMA_32X32X16_MIX),
+                          ("mfma_16x16x32_f16_mix", pkg.BENCH_MFMA_16X16X32_MIX)):
+        flops = ctypes.c_double(0.0)
+
+        def launch():
+            st = lib.glm_bench_mfma(pattern, operands.data_ptr(), operands.numel() * 2, 2000, sink.data_ptr(), sh,
+                                    ctypes.byref(flops))
+            if st != 0:
+                pkg.check(st, "glm_bench_mfma")
+
+        with torch.cuda.stream(stream):
+            for _ in range(4):  # a few milliseconds each: the clock settles
+                launch()
+            torch.cuda.synchronize()
+            e0 = torch.cuda.Event(enable_timing=True)
+            e1 = torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            for _ in range(4):
+                launch()
+            e1.record(stream)
+            torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / 4
+        tf = flops.value / (ms * 1e-3) / 1e12
+        out[name] = {"ms_per_launch": round(ms, 3), "tflops": round(tf, 1),
+                     "frac_of_mfma_peak": round(tf / MFMA_FP16_PEAK_TFLOPS, 4)}
+    return out
+
+
 def timelines(torch, pkg, capi):
     """In-kernel clock readings of the instrumented build: the decode launch of the headline workload and causal
     prompts of the ChatGLM3-6B shape.  Times are us since the first wave of the launch started; reading the clock
@@ -242,6 +284,7 @@ def main():
     if args.ceiling:
         with optional_section(result, "ceiling"):
             result["ceiling"] = read_ceilings(torch, pkg, kv, layer_halfs, stream, args.warmup, args.steps)
+            result["ceiling"]["mfma"] = mfma_ceilings(torch, pkg, stream)
 
     # ------------------------------------------------------------------ decode
     if not args.prefill_only and not args.ceiling_only:
@@ -368,6 +411,63 @@ def main():
                            "vs_baseline": None, "dtype": "f16", "data": "synthetic",
                            "config": {"workload": result["prefill"]["workload"]},
                            "roofline": result["prefill"]["roofline"]})
+
+    # ------------------------------------------------------------------ causal prompt (BASELINE config 2)
+    if not args.skip_prefill and not args.prefill_only:
+        with optional_section(result, "prefill_causal_2048"):
+            c_layers, c_h, c_kvh, c_len, c_q = 4, 32, 2, 8192, 2048
+            ctx2 = pkg.Context(num_layers=c_layers, num_attention_heads=c_h, num_key_value_heads=c_kvh, head_size=D,
+                               max_length=c_len, max_qlen=c_q)
+            c_width = (c_h + 2 * c_kvh) * D
+            qkv_c = torch.randn(c_layers, c_q, c_width, generator=gen, device=dev, dtype=torch.float32)
+            out_c = torch.zeros(c_layers, c_q, c_h * D, device=dev, dtype=torch.float32)
+            pos_c = torch.arange(c_q, device=dev, dtype=torch.int32)
+
+            def c_forward():
+                for l in range(c_layers):
+                    st = ctx2.forward(l, qkv_c[l].data_ptr(), c_q, 0, out_c[l].data_ptr(),
+                                      position_ids_ptr=pos_c.data_ptr(), stream=sh)
+                    if st != 0:
+                        pkg.check(st, "glm_attn_forward")
+
+            def c_rope():
+                for l in range(c_layers):
+                    st = ctx2.rope_append(l, qkv_c[l].data_ptr(), pos_c.data_ptr(), c_q, 0, stream=sh)
+                    if st != 0:
+                        pkg.check(st, "glm_attn_rope_append")
+
+            def c_time(fn):
+                with torch.cuda.stream(stream):
+                    for _ in range(3):
+                        fn()
+                    torch.cuda.synchronize()
+                    e0 = torch.cuda.Event(enable_timing=True)
+                    e1 = torch.cuda.Event(enable_timing=True)
+                    e0.record(stream)
+                    for _ in range(10):
+                        fn()
+                    e1.record(stream)
+                    torch.cuda.synchronize()
+                return e0.elapsed_time(e1) * 1e3 / (10 * c_layers)  # us per layer
+
+            us_call, us_rope = c_time(c_forward), c_time(c_rope)
+            assert bool(torch.isfinite(out_c).all()), "causal prompt produced non-finite output"
+            c_flops = 4 * c_h * D * (c_q * (c_q + 1) // 2)
+            us_kernel = us_call - us_rope
+            result["prefill_causal_2048"] = {
+                "workload": "ChatGLM3-6B shape (32 heads, 2 KV groups, max_length 8192): one 2048-token chunk at "
+                            "n_past=0, causal, per layer",
+                "us_per_layer": round(us_call, 2),
+                "rope_append_us": round(us_rope, 2),
+                "tokens_per_s": round(c_q / (us_call * 1e-6), 1),
+                "tflops_whole_call": round(c_flops / us_call / 1e6, 1),
+                "roofline": {"bound": "mfma", "kernel": "prefill_kernel",
+                             "duration": "the call minus rope_append_kernel timed alone (both launches of the call)",
+                             "achieved": round(c_flops / us_kernel / 1e6, 1), "peak": MFMA_FP16_PEAK_TFLOPS,
+                             "unit": "TFLOP/s", "frac": round(c_flops / us_kernel / 1e6 / MFMA_FP16_PEAK_TFLOPS, 4),
+                             "flops_per_launch": c_flops},
+            }
+            ctx2.close()
 
     # ------------------------------------------------------------------ the projections either side of the path
     if not args.skip_linear and not args.prefill_only:

@@ -40,7 +40,8 @@ MODEL_FILE_SYMBOLS = [
     "glm_model_file_data", "glm_model_file_tensor_count", "glm_model_file_tensor", "glm_model_file_find",
     "glm_model_file_upload",
 ]
-BENCH_SYMBOLS = ["glm_bench_read"]
+BENCH_SYMBOLS = ["glm_bench_mfma", "glm_bench_read"]
+BENCH_MFMA_32X32X16, BENCH_MFMA_16X16X32, BENCH_MFMA_32X32X16_MIX, BENCH_MFMA_16X16X32_MIX = 0, 1, 2, 3
 BENCH_READ_LINEAR, BENCH_READ_DECODE_PATTERN, BENCH_READ_STREAM, BENCH_EMPTY = 0, 1, 2, 3
 MODEL_F32, MODEL_F16, MODEL_Q4_0, MODEL_Q4_1, MODEL_Q5_0, MODEL_Q5_1, MODEL_Q8_0 = 0, 1, 2, 3, 6, 7, 8
 
@@ -284,6 +285,8 @@ def lib():
     L.glm_block_embedding.restype = c.c_int
     L.glm_bench_read.argtypes = [c.c_int, P, c.c_int32, c.c_int32, c.c_size_t, P, P]
     L.glm_bench_read.restype = c.c_int
+    L.glm_bench_mfma.argtypes = [c.c_int, P, c.c_size_t, c.c_int32, P, P, c.POINTER(c.c_double)]
+    L.glm_bench_mfma.restype = c.c_int
     L.glm_model_file_open.argtypes = [c.c_char_p, c.POINTER(P)]
     L.glm_model_file_open.restype = c.c_int
     L.glm_model_file_close.argtypes = [P]

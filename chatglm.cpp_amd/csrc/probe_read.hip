@@ -1,7 +1,7 @@
 // Read kernels that do nothing but load: what this GPU gives a launch shaped like the decode kernel's
 // (one workgroup per CU, every load of the launch issued up front), with the arithmetic, the exchange
-// between workgroups and the output taken away.  bench.py --ceiling times them; they are no part of the
-// attention path.
+// between workgroups and the output taken away; and loops of matrix instructions: what the matrix pipes give
+// the prefill kernel.  bench.py --ceiling times them; they are no part of the attention path.
 #include "glm_attn_internal.h"
 #include "glm_bench.h"
 
@@ -106,6 +106,135 @@ __global__ void empty_kernel(float *sink, int never) {
 }  // namespace glm_attn
 
 using namespace glm_attn;
+
+namespace glm_attn {
+namespace {
+
+// Loops of nothing but matrix instructions on operands with random bits, two waves per SIMD on every CU:
+// what the matrix pipes of this GPU sustain at the clock its power management grants them.
+//   SHAPE 0: v_mfma_f32_32x32x16_f16, four independent accumulators
+//   SHAPE 1: v_mfma_f32_16x16x32_f16, eight independent accumulators
+//   MIX    : the attention kernel's diet beside them: one 16-byte-per-lane LDS read per matrix instruction's
+//            worth of 32x32x16 work, and per four such instructions 21 vector instructions, 4 of them v_exp_f32
+template <int SHAPE, int MIX>
+__global__ __launch_bounds__(256, 2) void mfma_loop_kernel(const half8 *in, float *sink, int iters) {
+    __shared__ half8 lds[2048];  // 32 KiB
+    for (int i = threadIdx.x; i < 2048; i += 256) {
+        lds[i] = in[i];
+    }
+    __syncthreads();
+    const int lane = threadIdx.x & 63;
+    half8 a[4], b[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        a[i] = in[i * 64 + lane];
+        b[i] = in[256 + i * 64 + lane];
+    }
+    floatx16 c32[4];
+    floatx4 c16[8];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            c32[i][r] = 0.f;
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        c16[i] = floatx4{0.f, 0.f, 0.f, 0.f};
+    }
+    float v[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        v[i] = (float)in[512 + lane][i];
+    }
+    int at = lane;
+    for (int it = 0; it < iters; it++) {
+#pragma unroll
+        for (int g = 0; g < 8; g++) {
+            if (MIX) {
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    a[i] = lds[(at + g * 64 + i * 512) & 2047];
+                }
+            }
+            if (SHAPE == 0) {
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    c32[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[i], b[i], c32[i], 0, 0, 0);
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    c16[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[i >> 1], b[(i & 1) * 2 + (i >> 2)], c16[i], 0, 0, 0);
+                }
+            }
+            if (MIX) {
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    float x = __builtin_fmaf(v[e], 1.4426950f, -v[e + 4]);
+                    x = __builtin_amdgcn_exp2f(x);
+                    v[e + 4] = fmaxf(v[e + 4], x) * 0.5f;
+                    v[e] = __builtin_fmaf(v[e], 0.999f, x) + 0.001f;
+                }
+            }
+        }
+        at += 7;
+    }
+    float acc = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        acc += v[i] + c16[i][0] + c16[i][1] + c16[i][2] + c16[i][3];
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            acc += c32[i][r];
+        }
+    }
+    if (acc == 12345.678f) {
+        *sink = acc;
+    }
+}
+
+}  // namespace
+}  // namespace glm_attn
+
+extern "C" int glm_bench_mfma(int pattern, const void *operands, size_t operand_bytes, int32_t iters, float *sink,
+                              void *stream, double *flops) {
+    using namespace glm_attn;
+    if (!operands || !sink || iters <= 0 || operand_bytes < 2048 * sizeof(half8)) return GLM_ATTN_EINVAL;
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) {
+        return GLM_ATTN_EHIP;
+    }
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const half8 *in = static_cast<const half8 *>(operands);
+    const dim3 grid(2 * cus), block(256);
+    switch (pattern) {
+    case GLM_BENCH_MFMA_32X32X16:
+        hipLaunchKernelGGL((mfma_loop_kernel<0, 0>), grid, block, 0, st, in, sink, iters);
+        break;
+    case GLM_BENCH_MFMA_16X16X32:
+        hipLaunchKernelGGL((mfma_loop_kernel<1, 0>), grid, block, 0, st, in, sink, iters);
+        break;
+    case GLM_BENCH_MFMA_32X32X16_MIX:
+        hipLaunchKernelGGL((mfma_loop_kernel<0, 1>), grid, block, 0, st, in, sink, iters);
+        break;
+    case GLM_BENCH_MFMA_16X16X32_MIX:
+        hipLaunchKernelGGL((mfma_loop_kernel<1, 1>), grid, block, 0, st, in, sink, iters);
+        break;
+    default:
+        return GLM_ATTN_EINVAL;
+    }
+    if (flops) {
+        // per wave and iteration: 8 groups of 4 x 32x32x16 (or 8 x 16x16x32) = 8 x 131072 multiply-adds x 2
+        *flops = (double)grid.x * 4.0 * iters * 8.0 * 4.0 * 32.0 * 32.0 * 16.0 * 2.0;
+    }
+    return hipGetLastError() == hipSuccess ? GLM_ATTN_OK : GLM_ATTN_EHIP;
+}
 
 extern "C" int glm_bench_read(int pattern, const void *base, int32_t cache_rows, int32_t kv_heads, size_t bytes,
                               float *sink, void *stream) {

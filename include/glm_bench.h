@@ -1,7 +1,8 @@
 /*
  * Measurement aids of libglm_attn.so for `bench.py --ceiling`.  They have no counterpart in the reference
  * and are no part of the attention path: kernels that only load, shaped like a launch of the decode
- * kernel, so that the read rate this GPU gives such a launch can be measured beside the kernel's own.
+ * kernel, so that the read rate this GPU gives such a launch can be measured beside the kernel's own, and
+ * loops of matrix instructions, so that what the matrix pipes sustain can be measured beside the prefill kernel.
  */
 #ifndef GLM_BENCH_H
 #define GLM_BENCH_H
@@ -26,6 +27,21 @@ enum glm_bench_pattern {
    `sink` is a device float that is never written in practice.  Returns a glm_attn status. */
 int glm_bench_read(int pattern, const void *base, int32_t cache_rows, int32_t kv_heads, size_t bytes, float *sink,
                    void *stream);
+
+enum glm_bench_mfma_pattern {
+    GLM_BENCH_MFMA_32X32X16 = 0,     /* nothing but v_mfma_f32_32x32x16_f16, two waves per SIMD on every CU */
+    GLM_BENCH_MFMA_16X16X32 = 1,     /* nothing but v_mfma_f32_16x16x32_f16 */
+    GLM_BENCH_MFMA_32X32X16_MIX = 2, /* with the attention kernel's diet beside them: an LDS read of 16 bytes per
+                                        lane per 32x32x16 and 21 vector instructions (4 v_exp_f32) per four */
+    GLM_BENCH_MFMA_16X16X32_MIX = 3
+};
+
+/* Launches one loop of matrix instructions on `stream`: 2 workgroups of 4 waves per CU, `iters` iterations of
+   32 32x32x16 (or 64 16x16x32) instructions per wave.  `operands`: at least 32 KiB of device memory holding
+   fp16 values (finite ones, or the timing measures exception paths).  *flops (may be NULL) receives the
+   floating-point operations of the launch.  Returns a glm_attn status. */
+int glm_bench_mfma(int pattern, const void *operands, size_t operand_bytes, int32_t iters, float *sink, void *stream,
+                   double *flops);
 
 #ifdef __cplusplus
 }

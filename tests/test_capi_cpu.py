@@ -131,11 +131,12 @@ def test_library_exports_every_symbol_of_the_bench_header():
     lib = pkg.lib()
     names = declared_symbols("glm_bench.h", "glm_bench_")
     names = [n for n in names if n != "glm_bench_pattern"]
-    assert names == ["glm_bench_read"]
+    assert names == ["glm_bench_mfma", "glm_bench_read"]
     for n in names:
         assert hasattr(lib, n), f"{n} is declared in include/glm_bench.h but not exported"
     assert sorted(pkg.BENCH_SYMBOLS) == names
     assert lib.glm_bench_read(pkg.BENCH_READ_LINEAR, None, 256, 2, 0, None, None) == pkg.EINVAL
+    assert lib.glm_bench_mfma(pkg.BENCH_MFMA_32X32X16, None, 0, 1, None, None, None) == pkg.EINVAL
 
 
 def test_library_exports_every_symbol_of_the_model_file_header():
