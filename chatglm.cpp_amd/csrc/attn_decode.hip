@@ -499,10 +499,11 @@ __device__ inline int merge_quads(const MergeGeom &mg, int q_begin, int q_end, i
     return 0;
 }
 
-// Before its first look at the lines of the others a wave waits an eighth of its own run time so far plus
-// 0.3 us (see decode_body).
-constexpr int kFirstLookDiv = 8;
-constexpr int kFirstLookTicks = 30;  // of the 100 MHz clock
+// Before its first look at the lines of the others a wave waits 0.7 us plus 0.12 us per 4096 keys of the group
+// (see decode_body), in ticks of the 100 MHz clock.  Measured at 32767 keys: 1.0 us of waiting 11.7 us a layer,
+// 1.6 to 1.9 us 11.3 us, 2.2 us 11.6 us; at 4095 keys 0.8 us is the best.
+constexpr int kFirstLookTicks = 70;
+constexpr int kFirstLookTicksPer64Tiles = 12;
 constexpr int PPITCH = W * TILE + 8;  // row pitch of the P tile in LDS (halfs): conflict-free 16-byte accesses
 constexpr int kBlock = 2 * W * 64;    // W score waves, then W output waves
 
@@ -1021,11 +1022,14 @@ __device__ inline void decode_body(const DecodeArgs &a, DecodeShared &sh) {
         const unsigned long long t0 = wall_clock64();
         const unsigned long long limit = (unsigned long long)a.spin_ticks;
         // The lines are polled directly (a shared arrival counter would be one hot address for all the
-        // workgroups of a group).  Other workgroups finish up to a good fraction of this one's own run
-        // time later, and a line takes a while to become visible: looking right away would load nearly
-        // every line twice, so the first look waits a little.
+        // workgroups of a group).  Other workgroups finish later than this one by a time that grows with
+        // the bytes the launch moves, and a line takes a while to become visible: every look before the
+        // last line is there loads the missing ones again, and those loads compete with the tiles that
+        // slower workgroups are still waiting for.  So the first look waits.
         {
-            const unsigned long long wait_ticks = (t0 - ge.t_start) / kFirstLookDiv + kFirstLookTicks;
+            const int n_tiles = a.tiles_q * a.nsplit + a.tiles_r;
+            const unsigned long long wait_ticks =
+                (unsigned long long)(kFirstLookTicks + n_tiles * kFirstLookTicksPer64Tiles / 64);
             while (wall_clock64() - t0 < wait_ticks && wait_ticks < limit) {
                 __builtin_amdgcn_s_sleep(4);
             }
