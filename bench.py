@@ -26,7 +26,7 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
 # HBM bytes one decode_kernel launch of this workload moves, from two rocprofv3 --pmc runs of this script
-# (FETCH_SIZE 20,890 KiB x 2.000, WRITE_SIZE 2,273 KiB x 1.000; scales from a 256 MiB device copy in the same runs)
+# (FETCH_SIZE 17,783 KiB x 2.000, WRITE_SIZE 2,073 KiB x 1.000; scales from a 256 MiB device copy in the same runs)
 DECODE_TRAFFIC_BYTES_PER_LAUNCH = 38_540_000
 MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16
 
