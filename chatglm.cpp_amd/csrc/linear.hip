@@ -368,9 +368,12 @@ __global__ void gated_rows_f16_kernel(const float *x, const float *up, int activ
 // Y^T tile = W tile (features on MFMA rows) x X^T tile (input rows on MFMA columns).  Waves: 2 x 2, each
 // 64 features x 64 input rows = 2 x 2 blocks of 32 x 32.
 // `residual` (or null) has y's shape and may be y itself: a lane reads its 4 values right before it writes the same 4.
+// gridDim.z > 1 (a few rows against a weight with too few feature tiles to fill the chip): workgroup z takes share z
+// of the input features and leaves its sums, without bias or residual, in part[z][row][feature] for
+// splitk_reduce_kernel.
 __global__ __launch_bounds__(GM_THREADS, 2) void gemm_f16_kernel(const __half *W, const float *bias, const __half *x16,
                                                                  int rows, int K, int N, float *y, const float *residual,
-                                                                 float residual_scale) {
+                                                                 float residual_scale, float *part) {
     __shared__ __attribute__((aligned(1024))) __half Ws[2][GM_TILE][GM_K];
     __shared__ __attribute__((aligned(1024))) __half Xs[2][GM_TILE][GM_K];
     const int tid = threadIdx.x, lane = tid & 63;
@@ -390,7 +393,11 @@ __global__ __launch_bounds__(GM_THREADS, 2) void gemm_f16_kernel(const __half *W
             }
         }
     }
-    const int n_steps = K / GM_K;
+    const int ksplit = gridDim.z, kz = blockIdx.z;
+    const int step0 = (int)((int64_t)(K / GM_K) * kz / ksplit), step1 = (int)((int64_t)(K / GM_K) * (kz + 1) / ksplit);
+    const int n_steps = step1 - step0;
+    W += step0 * GM_K;
+    x16 += step0 * GM_K;
     gm_fetch(W, N, K, f0, 0, w, lane, Ws[0]);
     gm_fetch(x16, rows, K, r0, 0, w, lane, Xs[0]);
     for (int step = 0; step < n_steps; step++) {
@@ -435,6 +442,10 @@ __global__ __launch_bounds__(GM_THREADS, 2) void gemm_f16_kernel(const __half *W
                     if (f < N) {  // N is a multiple of 4 on this path
                         floatx4 v = {acc[fb][rb][4 * b4], acc[fb][rb][4 * b4 + 1], acc[fb][rb][4 * b4 + 2],
                                      acc[fb][rb][4 * b4 + 3]};
+                        if (ksplit > 1) {
+                            *reinterpret_cast<floatx4 *>(part + ((int64_t)kz * rows + row) * N + f) = v;
+                            continue;
+                        }
                         if (bias) {
                             v += *reinterpret_cast<const floatx4 *>(bias + f);
                         }
@@ -450,6 +461,29 @@ __global__ __launch_bounds__(GM_THREADS, 2) void gemm_f16_kernel(const __half *W
                 }
             }
         }
+    }
+}
+
+// y = sum over the shares of part (in the order of the shares) + bias + residual * scale, four values per thread
+__global__ void splitk_reduce_kernel(const float *part, int ksplit, int rows, int N, const float *bias,
+                                     const float *residual, float residual_scale, float *y) {
+    const int64_t n4 = (int64_t)rows * N / 4;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += (int64_t)gridDim.x * blockDim.x) {
+        floatx4 v = *reinterpret_cast<const floatx4 *>(part + i * 4);
+        for (int z = 1; z < ksplit; z++) {
+            v += *reinterpret_cast<const floatx4 *>(part + (int64_t)z * rows * N + i * 4);
+        }
+        if (bias) {
+            v += *reinterpret_cast<const floatx4 *>(bias + (i * 4) % N);
+        }
+        if (residual) {
+            const floatx4 r = *reinterpret_cast<const floatx4 *>(residual + i * 4);
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                v[e] = __fadd_rn(v[e], __fmul_rn(r[e], residual_scale));
+            }
+        }
+        *reinterpret_cast<floatx4 *>(y + i * 4) = v;
     }
 }
 
@@ -508,6 +542,10 @@ static RowStaging g_staging[64];
 // Likewise one fp16 buffer per device that a block-quantised weight is expanded into ahead of a GEMM, as large as
 // the largest quantised weight of the layers created on the device so far.
 static RowStaging g_dequant[64];
+// And one fp32 buffer per device for the shares of a GEMM that is cut along the input features (a few rows
+// against a weight with fewer feature tiles than the GPU has CUs): kSplitKMax x 128 rows x out_features.
+static RowStaging g_splitk[64];
+constexpr int kSplitKMax = 8;
 static std::mutex g_lt_mutex;
 static LtDevice g_lt[64];
 
@@ -533,6 +571,7 @@ struct glm_linear {
     bool committed;
     glm_attn::QuantPlanes q;
     RowStaging *dequant;  // the device's fp16 expansion buffer (quantised weights only)
+    RowStaging *splitk;   // the device's buffer for the shares of a GEMM cut along the input features, or null
     int max_rows;
     int last_hip_error;
 };
@@ -688,6 +727,7 @@ int glm_linear_create(const glm_linear_desc *desc, glm_linear **out_linear) {
     l->owns_weight = l->owns_bias = false;
     l->staging = nullptr;
     l->dequant = nullptr;
+    l->splitk = nullptr;
     l->quant = quant;
     l->committed = !quant;
     memset(&l->q, 0, sizeof(l->q));
@@ -756,6 +796,11 @@ int glm_linear_create(const glm_linear_desc *desc, glm_linear **out_linear) {
             std::lock_guard<std::mutex> lock(g_lt_mutex);
             LINEAR_TRY(grow(g_staging[desc->device], sizeof(__half) * (size_t)l->max_rows * (size_t)desc->in_features));
             l->staging = &g_staging[desc->device];
+            if ((desc->out_features + glm_attn::GM_TILE - 1) / glm_attn::GM_TILE < l->num_cus) {
+                const size_t r = l->max_rows < glm_attn::GM_TILE ? l->max_rows : glm_attn::GM_TILE;
+                LINEAR_TRY(grow(g_splitk[desc->device], sizeof(float) * kSplitKMax * r * (size_t)desc->out_features));
+                l->splitk = &g_splitk[desc->device];
+            }
         }
     }
     if ((desc->weight_dtype == GLM_LINEAR_F16 || quant) && l->max_rows > 8) {
@@ -958,9 +1003,27 @@ static int linear_forward_impl(glm_linear *l, glm_linear *l2, const glm_linear_f
             }
         }
         if (!done) {
-            hipLaunchKernelGGL(gemm_f16_kernel, dim3((N + GM_TILE - 1) / GM_TILE, (rows + GM_TILE - 1) / GM_TILE),
-                               dim3(GM_THREADS), 0, stream, static_cast<const __half *>(weight), l->bias, l->staging->x16,
-                               rows, K, N, y, residual, residual ? fu->residual_scale : 0.f);
+            // One tile of rows against fewer feature tiles than CUs: cut along the input features as well, so
+            // that the weight is streamed by the whole chip (a prompt of 20 tokens is bound by that stream).
+            const int f_tiles = (N + GM_TILE - 1) / GM_TILE;
+            int ksplit = 1;
+            if (rows <= GM_TILE && l->splitk && f_tiles < l->num_cus) {
+                ksplit = l->num_cus / f_tiles;
+                if (ksplit > kSplitKMax) ksplit = kSplitKMax;
+                if (ksplit > K / GM_K) ksplit = K / GM_K;
+                if (sizeof(float) * (size_t)ksplit * (size_t)rows * (size_t)N > l->splitk->bytes) ksplit = 1;
+            }
+            const float rscale = residual ? fu->residual_scale : 0.f;
+            float *part = ksplit > 1 ? reinterpret_cast<float *>(l->splitk->x16) : nullptr;
+            hipLaunchKernelGGL(gemm_f16_kernel, dim3(f_tiles, (rows + GM_TILE - 1) / GM_TILE, ksplit), dim3(GM_THREADS), 0,
+                               stream, static_cast<const __half *>(weight), l->bias, l->staging->x16, rows, K, N, y,
+                               residual, rscale, part);
+            if (ksplit > 1) {
+                const int64_t o4 = (int64_t)rows * N / 4;
+                const int rb = (int)((o4 + 255) / 256 < 1024 ? (o4 + 255) / 256 : 1024);
+                hipLaunchKernelGGL(splitk_reduce_kernel, dim3(rb), dim3(256), 0, stream, part, ksplit, rows, N, l->bias,
+                                   residual, rscale, y);
+            }
         }
     } else {
         const int64_t n_out = (int64_t)rows * N;
