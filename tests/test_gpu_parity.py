@@ -259,8 +259,8 @@ def test_range_errors(H):
 
 @pytest.mark.parametrize("n_past", [700, 2047])
 def test_decode_slow_path_when_workgroups_do_not_wait(H, n_past):
-    """With a zero wait bound every workgroup but the last leaves the hand-over at once and the last
-    arriver merges all slices: the result must not change."""
+    """With a zero wait bound a wave gives up on its first look, flags its slice and looks once more; slices that
+    are still missing then are redone by the workgroups that finish later: the result must not change."""
     p = H.Pair(max_length=2048)
     p.ctx.set_spin_limit_us(0)
     p.fill_past(0, n_past, seed=n_past)
@@ -270,6 +270,7 @@ def test_decode_slow_path_when_workgroups_do_not_wait(H, n_past):
         out, ref, _ = p.forward(0, qkv, n_past, host_pos=True, entry="decode")
         p.assert_caches_equal(0, "slow path")
         H.assert_close(out, ref, f"slow path rep {rep}")
+    assert p.ctx.device_flags() == 0  # every slice was written in the end, by its owner's second look or by a sweep
     p.close()
 
 
@@ -291,8 +292,11 @@ def test_decode_repeated_launches_reuse_the_handover_state(H):
 # The merge across workgroups changes shape with the number of splits (lanes per record 1..64, one wave or
 # several per quad of records, one or two batches of splits) and with the group size (padding heads).
 @pytest.mark.parametrize("h,kvh,max_length,n_past", [
-    (32, 2, 8192, 100),    # 2 splits
-    (32, 2, 8192, 200),    # 4
+    (32, 2, 8192, 100),    # 2 tiles: one workgroup per group, no exchange
+    (32, 2, 8192, 200),    # 4 tiles: the same, a full round
+    (32, 2, 8192, 300),    # 5 splits of one tile
+    (128, 128, 1024, 600), # 2 splits (2 CUs per group) of 5 tiles: two rounds in a workgroup
+    (64, 64, 2048, 1000),  # 4 splits of 4 tiles
     (32, 2, 8192, 500),    # 8
     (32, 2, 8192, 1000),   # 16
     (32, 2, 8192, 1500),   # 24
@@ -313,6 +317,7 @@ def test_decode_merge_geometries(H, h, kvh, max_length, n_past):
         out, ref, _ = p.forward(0, qkv, n_past, host_pos=True, entry="decode")
         p.assert_caches_equal(0, f"decode h={h} kvh={kvh} n_past={n_past}")
         H.assert_close(out, ref, f"decode h={h} kvh={kvh} n_past={n_past} rep {rep}")
+    assert p.ctx.device_flags() == 0
     p.close()
 
 
@@ -326,4 +331,5 @@ def test_decode_slow_path_geometries(H, n_past):
         out, ref, _ = p.forward(0, qkv, n_past, host_pos=True, entry="decode")
         p.assert_caches_equal(0, "slow path")
         H.assert_close(out, ref, f"slow path n_past={n_past} rep {rep}")
+    assert p.ctx.device_flags() == 0
     p.close()
