@@ -808,8 +808,11 @@ __device__ inline void score_wave(const DecodeArgs &a, DecodeShared &sh, const G
 
 // ---- output waves: O^T of 32 output dims over all keys of the workgroup.  Returns the lane's O (dims
 // w*32 + jb*16 + c*4 .. of head j), the head's sum and running max.
+// while_waiting(): work of the caller that needs the launch count but not the probabilities; it runs between the
+// issue of the V loads and the wait for the first probabilities, when the wave has nothing else to do.
+template <typename F>
 __device__ inline void output_wave(const DecodeArgs &a, DecodeShared &sh, const Geom &ge, floatx4 (&o)[2],
-                                   float &l_tot, float &m_fin) {
+                                   float &l_tot, float &m_fin, F while_waiting) {
     const int lane = ge.lane, w = ge.w, j = ge.j, c = ge.c, g = ge.g;
     const int L = a.s.L;
     const __half *Vg = a.v_cache + (int64_t)g * D * L;
@@ -849,6 +852,7 @@ __device__ inline void output_wave(const DecodeArgs &a, DecodeShared &sh, const 
     }
     TS(0);
     pin_value(ge.gen_v);  // nothing to do before P anyway
+    while_waiting();
     o[0] = floatx4{0.f, 0.f, 0.f, 0.f};
     o[1] = floatx4{0.f, 0.f, 0.f, 0.f};
     float m_run = -INFINITY;
@@ -1059,8 +1063,7 @@ __device__ inline void decode_body(const DecodeArgs &a, DecodeShared &sh) {
 
     floatx4 o[2];
     float l_tot, m_fin;
-    output_wave(a, sh, ge, o, l_tot, m_fin);
-    resolve();
+    output_wave(a, sh, ge, o, l_tot, m_fin, resolve);
     if (a.nsplit == 1) {
         // a single workgroup saw every key of the group: normalise and finish
         if (j < G) {
