@@ -665,6 +665,11 @@ hipError_t launch_prefill(const AttendArgs &a, int num_cus, hipStream_t stream) 
         while (nsplit > 1 && (int64_t)nsplit * n_qtiles * BM * units * (D + 2) > a.split_floats) nsplit--;
         if (nsplit < 2) nsplit = 1;
     }
+    // the partials of a cut launch must fit the scratch whatever chose nsplit (a launch that does not would write
+    // past it: checked here, on the host, once more)
+    if (nsplit > 1 && (!a.split_scratch || (int64_t)nsplit * n_qtiles * BM * units * (D + 2) > a.split_floats)) {
+        return hipErrorInvalidValue;
+    }
     if (two_groups) {
         hipLaunchKernelGGL(prefill_kernel<2>, dim3(n_items, nsplit), dim3(2 * THREADS), 0, stream, a, n_qtiles, order,
                            packed);
