@@ -945,10 +945,7 @@ __device__ inline void decode_body(const DecodeArgs &a, DecodeShared &sh) {
     const int lane = ge.lane, w = ge.w, j = ge.j, c = ge.c, g = ge.g, split = ge.split;
     const int G = a.s.G;
     // tiles [tb, te) of the keys already in the cache are this workgroup's
-    // (the last tiles_r splits take one tile more)
-    const int extra_from = a.nsplit - a.tiles_r;
-    ge.tb = split * a.tiles_q + (split > extra_from ? split - extra_from : 0);
-    ge.te = ge.tb + a.tiles_q + (split >= extra_from ? 1 : 0);
+    decode_tile_range(a.nsplit, a.tiles_q, a.tiles_r, split, &ge.tb, &ge.te);
     ge.rounds = ge.te - ge.tb > W ? (ge.te - ge.tb + W - 1) / W : 1;
     // The first workgroup also appends the new token and attends to it: every merge waits for its lines,
     // so it is the one that is dispatched first and never has the extra tile.

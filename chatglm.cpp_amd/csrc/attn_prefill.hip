@@ -44,12 +44,11 @@ extern "C" int glm_attn_debug_prefill_timeline(unsigned long long *host, size_t 
 namespace {
 
 constexpr int D = kFastHeadSize;
-constexpr int BM = 128;      // tokens per workgroup
-constexpr int BN = 64;       // keys per tile
+constexpr int BM = kPrefillRows;      // tokens per workgroup
+constexpr int BN = kPrefillTileKeys;  // keys per tile
 constexpr int WAVES = 4;
 constexpr int THREADS = WAVES * 64;
 constexpr float LOG2E = 1.4426950408889634f;
-constexpr int kPrefillMaxSplits = 128;
 constexpr int RING = 3;  // LDS fragments in flight ahead of the MFMAs (4 no longer fit the 256 registers)
 constexpr float kLazy = 8.f;  // see the online softmax in the kernel
 
@@ -634,52 +633,27 @@ __global__ __launch_bounds__(256) void merge_splits_kernel(AttendArgs a, int pad
 }  // namespace
 
 hipError_t launch_prefill(const AttendArgs &a, int num_cus, hipStream_t stream) {
-    // Up to 64 tokens of a grouped-query model are packed with the heads of their group (see the kernel): at
-    // least two heads then share every K/V tile.
-    const int packed = (a.s.G > 1 && a.qlen <= BM / 2) ? 1 : 0;
-    const int heads_per_unit = packed ? a.s.G : 1;
-    const int units = a.s.h / heads_per_unit;
-    const int rows = heads_per_unit * a.qlen;
-    const int n_qtiles = (rows + BM - 1) / BM;
-    const int n_items = n_qtiles * units;
-    // Too few items to give every CU two workgroups: eight-wave workgroups, one per CU (see the kernel).  Measured
-    // on 2048 causal tokens of 32 heads (512 items, 2 to 32 tiles each): 58 us with two four-wave workgroups per
-    // CU, 65 us with one of eight waves (nothing runs beside an item's first tiles and its last stores); on 1024
-    // tokens 29 us against 60 us for four-wave workgroups cut along the keys and merged by a second kernel.
-    const bool two_groups = n_items < 2 * num_cus;
-    const int slots = two_groups ? num_cus : 2 * num_cus;
-    const int order = (!a.causal || packed) ? 0 : (!two_groups && n_items == 2 * num_cus ? 2 : 1);
-    // A few tokens against a long cache are a handful of workgroups with hundreds of tiles each: cut the key
-    // range so that the chip is full once, as long as every share keeps at least four tiles per group of waves
-    // and the partials fit the scratch.
-    int nsplit = 1;
-    if (a.split_scratch && n_items < slots) {
-        int kv_end = a.kvs;
-        const int t_max = packed ? a.qlen : n_qtiles * BM;  // one past the last token of the last tile (or beyond)
-        if (a.causal && a.p0 + t_max < kv_end) kv_end = a.p0 + t_max;
-        const int n_tiles = (kv_end + BN - 1) / BN;
-        const int min_tiles = two_groups ? 8 : 4;
-        nsplit = (slots + n_items - 1) / n_items;
-        if (nsplit > n_tiles / min_tiles) nsplit = n_tiles / min_tiles;
-        if (nsplit > kPrefillMaxSplits) nsplit = kPrefillMaxSplits;
-        while (nsplit > 1 && (int64_t)nsplit * n_qtiles * BM * units * (D + 2) > a.split_floats) nsplit--;
-        if (nsplit < 2) nsplit = 1;
-    }
-    // the partials of a cut launch must fit the scratch whatever chose nsplit (a launch that does not would write
-    // past it: checked here, on the host, once more)
-    if (nsplit > 1 && (!a.split_scratch || (int64_t)nsplit * n_qtiles * BM * units * (D + 2) > a.split_floats)) {
+    // Measured on 2048 causal tokens of 32 heads (512 items, 2 to 32 tiles each): 58 us with two four-wave
+    // workgroups per CU, 65 us with one of eight waves (nothing runs beside an item's first tiles and its last
+    // stores); on 1024 tokens 29 us against 60 us for four-wave workgroups cut along the keys and merged by a
+    // second kernel.
+    const PrefillPlan pl = plan_prefill(a.qlen, a.p0, a.kvs, a.s.h, a.s.G, a.causal, a.split_scratch ? a.split_floats : 0,
+                                        num_cus);
+    // the partials of a cut launch must fit the scratch (a launch that does not would write past it: checked here
+    // once more, whatever chose nsplit)
+    if (pl.nsplit > 1 && (!a.split_scratch || pl.part_floats > a.split_floats)) {
         return hipErrorInvalidValue;
     }
-    if (two_groups) {
-        hipLaunchKernelGGL(prefill_kernel<2>, dim3(n_items, nsplit), dim3(2 * THREADS), 0, stream, a, n_qtiles, order,
-                           packed);
+    if (pl.two_groups) {
+        hipLaunchKernelGGL(prefill_kernel<2>, dim3(pl.n_items, pl.nsplit), dim3(2 * THREADS), 0, stream, a, pl.n_qtiles,
+                           pl.order, pl.packed);
     } else {
-        hipLaunchKernelGGL(prefill_kernel<1>, dim3(n_items, nsplit), dim3(THREADS), 0, stream, a, n_qtiles, order,
-                           packed);
+        hipLaunchKernelGGL(prefill_kernel<1>, dim3(pl.n_items, pl.nsplit), dim3(THREADS), 0, stream, a, pl.n_qtiles,
+                           pl.order, pl.packed);
     }
-    if (nsplit > 1) {
-        hipLaunchKernelGGL(merge_splits_kernel, dim3((unsigned)(((int64_t)rows * units + 7) / 8)), dim3(256), 0, stream, a,
-                           n_qtiles * BM, nsplit, packed);
+    if (pl.nsplit > 1) {
+        hipLaunchKernelGGL(merge_splits_kernel, dim3((unsigned)(((int64_t)pl.rows * pl.units + 7) / 8)), dim3(256), 0, stream,
+                           a, pl.n_qtiles * BM, pl.nsplit, pl.packed);
     }
     return hipGetLastError();
 }

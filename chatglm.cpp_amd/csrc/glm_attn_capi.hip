@@ -278,20 +278,10 @@ int do_decode(glm_attn_ctx *c, int layer, const float *qkv, const int32_t *posit
     da.scale = c->scale;
     da.k_cache = layer_k(c, layer);
     da.v_cache = layer_v(c, layer);
-    // Deal the 64-key tiles of a group out to as many workgroups as there are CUs for it: spreading
-    // over CUs first buys more load queues.  A workgroup takes its tiles four at a time.
-    const int n_tiles = (da.p0 + kDecodeTileKeys - 1) / kDecodeTileKeys;
-    const int cu_share = c->num_cus / c->shape.kvh > 0 ? c->num_cus / c->shape.kvh : 1;
-    int nsplit = n_tiles < 1 ? 1 : n_tiles;
-    if (nsplit > cu_share) nsplit = cu_share;
-    if (nsplit > c->max_splits) nsplit = c->max_splits;
-    if (shared && nsplit > kStaticMaxParts / c->shape.kvh) nsplit = kStaticMaxParts / c->shape.kvh;
-    // One round of tiles is over sooner in one workgroup than the exchange between several takes (a second
-    // round in the same workgroup is not: it costs 3 us, the exchange 2).
-    if (n_tiles <= kDecodeMaxWaves) nsplit = 1;
-    da.nsplit = nsplit;
-    da.tiles_q = n_tiles / nsplit;
-    da.tiles_r = n_tiles % nsplit;
+    const DecodePlan pl = plan_decode(da.p0, c->shape.kvh, c->num_cus, c->max_splits, shared ? kStaticMaxParts : 0);
+    da.nsplit = pl.nsplit;
+    da.tiles_q = pl.tiles_q;
+    da.tiles_r = pl.tiles_r;
     da.part = shared ? shared->part : c->part;
     da.out = out;
     da.flags = c->flags;

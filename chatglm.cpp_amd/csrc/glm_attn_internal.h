@@ -50,6 +50,88 @@ __host__ __device__ inline unsigned long long decode_next_gen(unsigned long long
     return decode_stamp(next) == 0u ? next + 1ull : next;
 }
 
+// ---- launch geometry, worked out on the host (plain functions, so that a host test can walk the shapes and
+// check every extent against what the launch is given)
+
+// decode_kernel: the 64-key tiles of the keys already in the cache, dealt out to nsplit workgroups per KV group
+// (tiles_q each, the last tiles_r one more).  max_parts: (group, split) partials the exchange memory holds.
+struct DecodePlan {
+    int n_tiles, nsplit, tiles_q, tiles_r;
+};
+inline DecodePlan plan_decode(int p0, int kvh, int num_cus, int max_splits, int max_parts) {
+    DecodePlan pl;
+    pl.n_tiles = (p0 + kDecodeTileKeys - 1) / kDecodeTileKeys;
+    // spread over CUs first: that buys more load queues; a workgroup takes its tiles four at a time
+    const int cu_share = num_cus / kvh > 0 ? num_cus / kvh : 1;
+    int nsplit = pl.n_tiles < 1 ? 1 : pl.n_tiles;
+    if (nsplit > cu_share) nsplit = cu_share;
+    if (nsplit > max_splits) nsplit = max_splits;
+    if (nsplit > kDecodeMaxSplits) nsplit = kDecodeMaxSplits;
+    if (max_parts > 0 && nsplit > max_parts / kvh) nsplit = max_parts / kvh;
+    // One round of tiles is over sooner in one workgroup than the exchange between several takes (a second
+    // round in the same workgroup is not: it costs 3 us, the exchange 2).
+    if (pl.n_tiles <= kDecodeMaxWaves) nsplit = 1;
+    if (nsplit < 1) nsplit = 1;
+    pl.nsplit = nsplit;
+    pl.tiles_q = pl.n_tiles / nsplit;
+    pl.tiles_r = pl.n_tiles % nsplit;
+    return pl;
+}
+
+// tiles [*tb, *te) of workgroup `split`: the last tiles_r splits take one tile more (the first workgroup, which
+// also appends the new token, never has the extra tile)
+__host__ __device__ inline void decode_tile_range(int nsplit, int tiles_q, int tiles_r, int split, int *tb, int *te) {
+    const int extra_from = nsplit - tiles_r;
+    *tb = split * tiles_q + (split > extra_from ? split - extra_from : 0);
+    *te = *tb + tiles_q + (split >= extra_from ? 1 : 0);
+}
+
+// prefill_kernel: rows of 128 per item, items of one unit (a head, or a KV group when a few tokens are packed with
+// the heads of their group), four-wave or eight-wave workgroups, and the cut along the keys with its partials.
+constexpr int kPrefillRows = 128;        // rows (tokens) per workgroup
+constexpr int kPrefillTileKeys = 64;     // keys per tile
+constexpr int kPrefillMaxSplits = 128;   // shares of the key range
+struct PrefillPlan {
+    int packed, units, rows, n_qtiles, n_items;
+    int two_groups, order, nsplit;
+    int64_t part_floats;  // floats of the partials of a cut launch (0 when nsplit == 1)
+};
+inline PrefillPlan plan_prefill(int qlen, int p0, int kvs, int h, int G, int causal, int64_t split_floats, int num_cus) {
+    PrefillPlan pl;
+    const int D = kFastHeadSize, BM = kPrefillRows, BN = kPrefillTileKeys;
+    // Up to 64 tokens of a grouped-query model are packed with the heads of their group: at least two heads then
+    // share every K/V tile.
+    pl.packed = (G > 1 && qlen <= BM / 2) ? 1 : 0;
+    const int heads_per_unit = pl.packed ? G : 1;
+    pl.units = h / heads_per_unit;
+    pl.rows = heads_per_unit * qlen;
+    pl.n_qtiles = (pl.rows + BM - 1) / BM;
+    pl.n_items = pl.n_qtiles * pl.units;
+    // Too few items to give every CU two workgroups: eight-wave workgroups, one per CU.
+    pl.two_groups = pl.n_items < 2 * num_cus ? 1 : 0;
+    const int slots = pl.two_groups ? num_cus : 2 * num_cus;
+    pl.order = (!causal || pl.packed) ? 0 : (!pl.two_groups && pl.n_items == 2 * num_cus ? 2 : 1);
+    // A few tokens against a long cache are a handful of workgroups with hundreds of tiles each: cut the key
+    // range so that the chip is full once, as long as every share keeps at least four tiles per group of waves
+    // and the partials fit the scratch.
+    int nsplit = 1;
+    if (split_floats > 0 && pl.n_items < slots) {
+        int kv_end = kvs;
+        const int t_max = pl.packed ? qlen : pl.n_qtiles * BM;  // one past the last token of the last tile (or beyond)
+        if (causal && p0 + t_max < kv_end) kv_end = p0 + t_max;
+        const int n_tiles = (kv_end + BN - 1) / BN;
+        const int min_tiles = pl.two_groups ? 8 : 4;
+        nsplit = (slots + pl.n_items - 1) / pl.n_items;
+        if (nsplit > n_tiles / min_tiles) nsplit = n_tiles / min_tiles;
+        if (nsplit > kPrefillMaxSplits) nsplit = kPrefillMaxSplits;
+        while (nsplit > 1 && (int64_t)nsplit * pl.n_qtiles * BM * pl.units * (D + 2) > split_floats) nsplit--;
+        if (nsplit < 2) nsplit = 1;
+    }
+    pl.nsplit = nsplit;
+    pl.part_floats = nsplit > 1 ? (int64_t)nsplit * pl.n_qtiles * BM * pl.units * (D + 2) : 0;
+    return pl;
+}
+
 // Where q, k and v heads sit inside one token's row of the fused projection (chatglm.cpp:636-653).
 struct QkvLayout {
     int64_t row_stride;  // floats between tokens

@@ -162,3 +162,18 @@ def test_decode_launch_stamps_on_the_host(tmp_path):
                    check=True, capture_output=True)
     out = subprocess.run([exe], capture_output=True, text=True)
     assert out.returncode == 0 and out.stdout.strip() == "ok", out.stdout + out.stderr
+
+
+def test_launch_geometry_on_the_host(tmp_path):
+    """tests/cpp/test_launch_plans.cpp: the functions that choose the grids of the decode and prefill kernels
+    (splits, tiles per workgroup, shares of the key range, partials), compiled for the host from the kernels' own
+    header and walked over many shapes: every extent a launch derives from them stays inside its buffer."""
+    import subprocess
+
+    exe = str(tmp_path / "test_launch_plans")
+    src = os.path.join(ROOT, "tests", "cpp", "test_launch_plans.cpp")
+    inc = ["-I" + os.path.join(ROOT, "include"), "-I" + os.path.join(ROOT, "chatglm.cpp_amd", "csrc")]
+    subprocess.run(["/opt/rocm/bin/hipcc", "-O1", "-std=c++17", "-x", "hip", "--offload-arch=gfx950", src, "-o", exe] + inc,
+                   check=True, capture_output=True)
+    out = subprocess.run([exe], capture_output=True, text=True)
+    assert out.returncode == 0 and out.stdout.strip() == "ok", out.stdout + out.stderr
