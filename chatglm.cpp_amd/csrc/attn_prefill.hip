@@ -50,7 +50,7 @@ constexpr int WAVES = 4;
 constexpr int THREADS = WAVES * 64;
 constexpr float LOG2E = 1.4426950408889634f;
 constexpr int RING = 3;  // LDS fragments in flight ahead of the MFMAs (4 no longer fit the 256 registers)
-constexpr float kLazy = 8.f;  // see the online softmax in the kernel
+constexpr float kLazy = 8.f / LOG2E;  // see the online softmax in the kernel: 8 in base-2 logarithm units
 
 typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 
@@ -314,7 +314,7 @@ __global__ __launch_bounds__(THREADS * GROUPS, 2 / GROUPS) void prefill_kernel(A
             o[db][r] = 0.f;
         }
     }
-    // Reference point of the exponentials for token n (log2 units, the same in both lane halves) and the sum of
+    // Reference point of the exponentials for token n (in the scores' units, the same in both lane halves) and the sum of
     // the probabilities of this lane's keys (the two halves of a token are added up after the last tile).
     float m = -INFINITY, l = 0.f;
     floatx16 nb;  // -m in every register (0 while m is -inf): where the score sums start
@@ -357,7 +357,7 @@ __global__ __launch_bounds__(THREADS * GROUPS, 2 / GROUPS) void prefill_kernel(A
     // S^T = K Q^T - m for the K tile in buffer buf: two 32-key blocks.  The 16 fragments come through a ring, so
     // that a read is issued RING MFMAs before its use.  between(i) runs after step i.  The sums start from
     // nb, which holds minus the reference point of the exponentials in all its registers (the lane's token is the
-    // same for all of them): the scores leave the matrix pipe ready for v_exp_f32.
+    // same for all of them): a score leaves the matrix pipe one multiplication (by log2 e) away from v_exp_f32.
     auto first_product = [&](int buf, floatx16 (&s)[2], auto between) __attribute__((always_inline)) {
         half8 fr[RING];
 #pragma unroll
@@ -432,7 +432,7 @@ __global__ __launch_bounds__(THREADS * GROUPS, 2 / GROUPS) void prefill_kernel(A
                     const int key = key0 + kb * 32 + 16 * (b >> 1) + 8 * c + 4 * (b & 1) + (r & 3);
                     float v = sc[kb][r];
                     if (a.mask && key < a.kvs) {
-                        v = __builtin_fmaf(a.mask[(int64_t)t_abs * a.kvs + key], LOG2E, v);  // scores are in log2 units
+                        v += a.mask[(int64_t)t_abs * a.kvs + key];
                     }
                     if (key >= kv_lim || (a.causal && key > a.p0 + t_abs)) {
                         v = -INFINITY;
@@ -451,8 +451,8 @@ __global__ __launch_bounds__(THREADS * GROUPS, 2 / GROUPS) void prefill_kernel(A
         // K(T+2) between the MFMAs, one piece at a time (eight pieces issued in one go fill the memory
         // pipe's queue and hold the wave up).
         // Online softmax for token n (the two lane halves hold different keys of it): the reference point m
-        // of the exponentials only moves when the running maximum has grown by more than kLazy (in log2
-        // units): probabilities may then reach 2^kLazy, which fp16 holds with full relative precision, and
+        // of the exponentials only moves when the running maximum has grown by more than kLazy (8 in log2
+        // units): probabilities may then reach 2^8, which fp16 holds with full relative precision, and
         // the rescaling of the 64 accumulator registers becomes rare.
         float mx = -INFINITY;  // over the scores as they are: relative to m
 #pragma unroll
@@ -474,7 +474,7 @@ __global__ __launch_bounds__(THREADS * GROUPS, 2 / GROUPS) void prefill_kernel(A
         if (__builtin_amdgcn_ballot_w64(move) != 0) {
             // by how much the reference point rises (from 0 to the maximum for a token's first keys)
             const float d = (mx == -INFINITY) ? 0.f : (m == -INFINITY ? mx : fmaxf(mx, 0.f));
-            const float alpha = (m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(-d);
+            const float alpha = (m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(-d * LOG2E);
 #pragma unroll
             for (int db = 0; db < 4; db++) {
                 o[db] *= alpha;
@@ -501,7 +501,8 @@ __global__ __launch_bounds__(THREADS * GROUPS, 2 / GROUPS) void prefill_kernel(A
         for (int kb = 0; kb < 2; kb++) {
 #pragma unroll
             for (int r = 0; r < 16; r += 2) {
-                const half2v h = {(_Float16)__builtin_amdgcn_exp2f(sc[kb][r]), (_Float16)__builtin_amdgcn_exp2f(sc[kb][r + 1])};
+                const half2v h = {(_Float16)__builtin_amdgcn_exp2f(sc[kb][r] * LOG2E),
+                                  (_Float16)__builtin_amdgcn_exp2f(sc[kb][r + 1] * LOG2E)};
                 l = __builtin_amdgcn_fdot2(h, ones, l, false);
                 const int b = r >> 2;
                 pf[kb * 2 + (b >> 1)][4 * (b & 1) + (r & 3)] = h[0];
@@ -533,6 +534,7 @@ __global__ __launch_bounds__(THREADS * GROUPS, 2 / GROUPS) void prefill_kernel(A
     PTS(5);
 
     l = sum_of_halves(l);
+    m *= LOG2E;  // from here on in base-2 logarithm units, which is what the merges' exponentials take
     if (GROUPS > 1) {
         // ---- the second group's (m, l, O) into the first's: wave w of either holds the same rows in the same
         // lanes, so O goes through LDS register by register, 64 lanes side by side (the second group's own tile

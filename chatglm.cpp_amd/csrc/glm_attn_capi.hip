@@ -214,10 +214,8 @@ int stage_positions(glm_attn_ctx *c, const int32_t *position_ids, const int32_t 
     return GLM_ATTN_OK;
 }
 
-// for_mfma: the queries go to prefill_kernel, which wants them scaled into base-2 logarithm units as well (its
-// exponentials are v_exp_f32, a power of two); the generic kernel takes them with the softmax scale alone
 int do_rope_append(glm_attn_ctx *c, int layer, const float *qkv, int64_t row_stride, const int32_t *dev_pos, int qlen,
-                   int n_past, hipStream_t stream, bool for_mfma) {
+                   int n_past, hipStream_t stream) {
     RopeAppendArgs ra;
     ra.qkv = qkv;
     ra.lay = call_layout(c, row_stride);
@@ -226,7 +224,7 @@ int do_rope_append(glm_attn_ctx *c, int layer, const float *qkv, int64_t row_str
     ra.position_ids = dev_pos;
     ra.qlen = qlen;
     ra.p0 = c->desc.num_virtual_tokens + n_past;
-    ra.scale = for_mfma ? c->scale * 1.4426950408889634f : c->scale;
+    ra.scale = c->scale;
     ra.q16 = c->q16;
     ra.k_cache = layer_k(c, layer);
     ra.v_cache = layer_v(c, layer);
@@ -486,7 +484,7 @@ int glm_attn_rope_append(glm_attn_ctx *ctx, int32_t layer, const float *qkv, int
     if (rc != GLM_ATTN_OK) return rc;
     if (!qkv || (ctx->rope.pairs > 0 && !position_ids)) return GLM_ATTN_EINVAL;
     DeviceGuard guard(ctx->desc.device);
-    return do_rope_append(ctx, layer, qkv, qkv_row_stride, position_ids, qlen, n_past, (hipStream_t)stream, false);
+    return do_rope_append(ctx, layer, qkv, qkv_row_stride, position_ids, qlen, n_past, (hipStream_t)stream);
 }
 
 int glm_attn_decode(glm_attn_ctx *ctx, int32_t layer, const float *qkv, const int32_t *position_ids,
@@ -525,7 +523,7 @@ int glm_attn_prefill(glm_attn_ctx *ctx, int32_t layer, const float *qkv, int64_t
     if (rc != GLM_ATTN_OK) return rc;
     DeviceGuard guard(ctx->desc.device);
     hipStream_t st = (hipStream_t)stream;
-    rc = do_rope_append(ctx, layer, qkv, qkv_row_stride, position_ids, qlen, n_past, st, true);
+    rc = do_rope_append(ctx, layer, qkv, qkv_row_stride, position_ids, qlen, n_past, st);
     if (rc != GLM_ATTN_OK) return rc;
     AttendArgs aa = make_attend(ctx, layer, qlen, n_past, causal, mask, out);
     HIP_TRY(ctx, launch_prefill(aa, ctx->num_cus, st));
@@ -554,7 +552,7 @@ int glm_attn_forward(glm_attn_ctx *ctx, int32_t layer, const float *qkv, int64_t
     rc = stage_positions(ctx, position_ids, position_ids_host, qlen, st, &dev_pos);
     if (rc != GLM_ATTN_OK) return rc;
     const bool mfma = ctx->fast && aligned16(out);
-    rc = do_rope_append(ctx, layer, qkv, qkv_row_stride, dev_pos, qlen, n_past, st, mfma);
+    rc = do_rope_append(ctx, layer, qkv, qkv_row_stride, dev_pos, qlen, n_past, st);
     if (rc != GLM_ATTN_OK) return rc;
     AttendArgs aa = make_attend(ctx, layer, qlen, n_past, causal, mask, out);
     if (mfma) {
