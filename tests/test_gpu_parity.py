@@ -289,8 +289,8 @@ def test_decode_repeated_launches_reuse_the_handover_state(H):
     p.close()
 
 
-# The merge across workgroups changes shape with the number of splits (lanes per record 1..64, one wave or
-# several per quad of records, one or two batches of splits) and with the group size (padding heads).
+# The merge across workgroups changes shape with the number of splits (split lanes per line 1..16, 1, 2, 4 or 8
+# lines per lane, one wave per quad or all four on one, one or two passes) and with the group size (padding heads).
 @pytest.mark.parametrize("h,kvh,max_length,n_past", [
     (32, 2, 8192, 100),    # 2 tiles: one workgroup per group, no exchange
     (32, 2, 8192, 200),    # 4 tiles: the same, a full round
@@ -311,7 +311,7 @@ def test_decode_repeated_launches_reuse_the_handover_state(H):
 def test_decode_merge_geometries(H, h, kvh, max_length, n_past):
     p = H.Pair(h=h, kvh=kvh, max_length=max_length, cache_fill=0x7E00)
     p.fill_past(0, n_past, seed=21 + n_past)
-    for rep in range(2):  # the second launch meets the first one's records in the exchange buffer
+    for rep in range(2):  # the second launch meets the first one's lines in the exchange buffer
         qkv = p.random_qkv(1, seed=600 + n_past + rep)
         p.fill_past(0, n_past, seed=21 + n_past)
         out, ref, _ = p.forward(0, qkv, n_past, host_pos=True, entry="decode")
