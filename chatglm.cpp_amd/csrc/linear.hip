@@ -21,6 +21,7 @@
 #include "glm_attn_internal.h"
 #include "glm_block.h"
 #include "glm_linear.h"
+#include "linear_plan.h"
 #include "linear_quant.h"
 
 namespace glm_attn {
@@ -280,8 +281,8 @@ __global__ __launch_bounds__(WAVES * 64, NBLK == 1 ? 4 : 2) void gemv_f16_kernel
 
 // ---------------------------------------------------------------- many rows: MFMA GEMM
 
-constexpr int GM_TILE = 128;  // output features and input rows per workgroup
-constexpr int GM_K = 64;      // input features per step
+constexpr int GM_TILE = kGemmTile;  // output features and input rows per workgroup
+constexpr int GM_K = kGemmK;        // input features per step
 constexpr int GM_WAVES = 4;
 constexpr int GM_THREADS = GM_WAVES * 64;
 
@@ -394,8 +395,12 @@ __global__ __launch_bounds__(GM_THREADS, 2) void gemm_f16_kernel(const __half *W
         }
     }
     const int ksplit = gridDim.z, kz = blockIdx.z;
-    const int step0 = (int)((int64_t)(K / GM_K) * kz / ksplit), step1 = (int)((int64_t)(K / GM_K) * (kz + 1) / ksplit);
+    int step0, step1;
+    splitk_step_range(K, ksplit, kz, &step0, &step1);
     const int n_steps = step1 - step0;
+    if (n_steps <= 0) {
+        return;  // (never: the host gives no share fewer than one step)
+    }
     W += step0 * GM_K;
     x16 += step0 * GM_K;
     gm_fetch(W, N, K, f0, 0, w, lane, Ws[0]);
@@ -545,7 +550,7 @@ static RowStaging g_dequant[64];
 // And one fp32 buffer per device for the shares of a GEMM that is cut along the input features (a few rows
 // against a weight with fewer feature tiles than the GPU has CUs): kSplitKMax x 128 rows x out_features.
 static RowStaging g_splitk[64];
-constexpr int kSplitKMax = 8;
+using glm_attn::kSplitKMax;
 static std::mutex g_lt_mutex;
 static LtDevice g_lt[64];
 
@@ -1006,13 +1011,7 @@ static int linear_forward_impl(glm_linear *l, glm_linear *l2, const glm_linear_f
             // One tile of rows against fewer feature tiles than CUs: cut along the input features as well, so
             // that the weight is streamed by the whole chip (a prompt of 20 tokens is bound by that stream).
             const int f_tiles = (N + GM_TILE - 1) / GM_TILE;
-            int ksplit = 1;
-            if (rows <= GM_TILE && l->splitk && f_tiles < l->num_cus) {
-                ksplit = l->num_cus / f_tiles;
-                if (ksplit > kSplitKMax) ksplit = kSplitKMax;
-                if (ksplit > K / GM_K) ksplit = K / GM_K;
-                if (sizeof(float) * (size_t)ksplit * (size_t)rows * (size_t)N > l->splitk->bytes) ksplit = 1;
-            }
+            const int ksplit = plan_splitk(rows, N, K, l->num_cus, l->splitk ? l->splitk->bytes : 0);
             const float rscale = residual ? fu->residual_scale : 0.f;
             float *part = ksplit > 1 ? reinterpret_cast<float *>(l->splitk->x16) : nullptr;
             hipLaunchKernelGGL(gemm_f16_kernel, dim3(f_tiles, (rows + GM_TILE - 1) / GM_TILE, ksplit), dim3(GM_THREADS), 0,

@@ -8,6 +8,7 @@
 #include <vector>
 
 #include "glm_attn_internal.h"
+#include "linear_plan.h"
 
 using namespace glm_attn;
 
@@ -119,8 +120,40 @@ static int check_prefill() {
     return 0;
 }
 
+static int check_splitk() {
+    char what[160];
+    const int Ns[] = {4, 64, 128, 132, 4096, 4608, 13696, 27392, 32768, 151552};
+    const int Ks[] = {64, 128, 256, 1408, 4096, 13696};
+    for (int num_cus : {256, 304, 64}) {
+        for (int N : Ns) {
+            for (int K : Ks) {
+                for (int rows : {1, 8, 9, 20, 64, 127, 128, 129, 300, 2048}) {
+                    for (size_t scratch : {(size_t)0, (size_t)4096, sizeof(float) * kSplitKMax * 128 * (size_t)N}) {
+                        const int ks = plan_splitk(rows, N, K, num_cus, scratch);
+                        snprintf(what, sizeof(what), "splitk cus %d N %d K %d rows %d scratch %zu -> %d", num_cus, N, K, rows,
+                                 scratch, ks);
+                        CHECK(ks >= 1 && ks <= kSplitKMax && ks <= K / kGemmK);
+                        CHECK(ks == 1 || (rows <= kGemmTile && sizeof(float) * (size_t)ks * rows * N <= scratch));
+                        CHECK(ks <= 65535);  // gridDim.z
+                        int at = 0;
+                        for (int kz = 0; kz < ks; kz++) {
+                            int s0, s1;
+                            splitk_step_range(K, ks, kz, &s0, &s1);
+                            CHECK(s0 == at && s1 > s0);  // in order, none empty
+                            CHECK((int64_t)s1 * kGemmK <= K);  // the last fetch of a share ends inside a row
+                            at = s1;
+                        }
+                        CHECK(at == K / kGemmK);
+                    }
+                }
+            }
+        }
+    }
+    return 0;
+}
+
 int main() {
-    if (check_decode() || check_prefill()) return 1;
+    if (check_decode() || check_prefill() || check_splitk()) return 1;
     printf("ok\n");
     return 0;
 }
