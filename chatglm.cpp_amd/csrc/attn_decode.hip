@@ -521,10 +521,10 @@ struct DecodeShared {
     int p_ready;        // score waves that have left their part of P, over all rounds
     int p_done;         // output waves that are through with P, over all rounds
     int stored;         // output waves whose line stores have been performed
-    // the four score waves on one quad of the output: what each leaves for the first of them
+    // several score waves on one quad of the output: what each leaves for the first of them
     float red[W][4][8];  // per wave and piece: max, sum, O[4]
-    int red_ready;
-    int red_fail;
+    int red_ready[2];    // per quad of the workgroup's slice (one, or two with two waves each)
+    int red_fail[2];
 };
 
 // A wave waits for waves of its own workgroup (all resident by construction) through a counter in LDS.
@@ -560,17 +560,24 @@ __device__ inline float sum_over_c(float x) {
     return __uint_as_float(b[0]) + __uint_as_float(b[1]);
 }
 
-// The long-context shape: one quad per workgroup and many splits.  All four score waves work on the
-// quad, 64 split lanes in all, and the first of them finishes it from what the others leave in LDS.
-__device__ inline int merge_quad4(const MergeGeom &mg, DecodeShared &sh, int q, int wv, int lane,
-                                  unsigned long long t0, unsigned long long limit, uint32_t *flags) {
-    const int piece = lane & 3, s = wv * 16 + (lane >> 2);
+// Many splits and a slice of one or two quads: WPQ = 4 or 2 score waves work on a quad, 16 split lanes each, and
+// the first of them finishes it from what the others leave in LDS.  wv: the wave among the score waves; its quad is
+// q_begin + wv / WPQ (a wave whose quad lies beyond the slice has nothing to do).
+template <int WPQ>
+__device__ inline int merge_quad_shared(const MergeGeom &mg, DecodeShared &sh, int q_begin, int q_end, int wv, int lane,
+                                        unsigned long long t0, unsigned long long limit, uint32_t *flags) {
+    const int ql = wv / WPQ, sub = wv % WPQ;
+    const int q = q_begin + ql;
+    if (q >= q_end) {
+        return 0;
+    }
+    const int piece = lane & 3, s = sub * 16 + (lane >> 2);
     const int hd = q / QUADS, quad = q - hd * QUADS;
     const float *base = mg.part_g + ((int64_t)(hd * QUADS + quad) * mg.nsplit * 4 + piece) * 4;
     Fold acc = {-INFINITY, 0.f, floatx4{0.f, 0.f, 0.f, 0.f}};
     int failed = 0;
-    for (int b0 = 0; b0 < mg.nsplit && !failed; b0 += 8 * 64) {
-        failed = poll_lines(base, b0, b0 + s, 64, mg.nsplit, true, mg.stamp32, piece, t0, limit, acc);
+    for (int b0 = 0; b0 < mg.nsplit && !failed; b0 += 8 * 16 * WPQ) {
+        failed = poll_lines(base, b0, b0 + s, 16 * WPQ, mg.nsplit, true, mg.stamp32, piece, t0, limit, acc);
     }
     reduce_fold(acc, 4);
     TS(4);
@@ -580,33 +587,33 @@ __device__ inline int merge_quad4(const MergeGeom &mg, DecodeShared &sh, int q, 
         dst[1] = acc.w;
         *reinterpret_cast<floatx4 *>(dst + 4) = acc.o;
         if (failed) {
-            sh.red_fail = 1;
+            sh.red_fail[ql] = 1;
         }
     }
-    lds_signal(&sh.red_ready, lane);
-    if (wv != 0) {
+    lds_signal(&sh.red_ready[ql], lane);
+    if (sub != 0) {
         return failed;
     }
-    lds_wait_ge(&sh.red_ready, W, flags);
-    failed |= __hip_atomic_load(&sh.red_fail, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    lds_wait_ge(&sh.red_ready[ql], WPQ, flags);
+    failed |= __hip_atomic_load(&sh.red_fail[ql], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     if (failed) {
         return 1;
     }
     if (lane < 4) {
         float m_all = acc.m;
 #pragma unroll
-        for (int ww = 1; ww < W; ww++) {
-            m_all = fmaxf(m_all, sh.red[ww][piece][0]);
+        for (int ww = 1; ww < WPQ; ww++) {
+            m_all = fmaxf(m_all, sh.red[wv + ww][piece][0]);
         }
         float f = (acc.m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(acc.m - m_all);
         float wsum = acc.w * f;
         floatx4 osum = acc.o * f;
 #pragma unroll
-        for (int ww = 1; ww < W; ww++) {
-            const float mw = sh.red[ww][piece][0];
+        for (int ww = 1; ww < WPQ; ww++) {
+            const float mw = sh.red[wv + ww][piece][0];
             f = (mw == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(mw - m_all);
-            wsum = __builtin_fmaf(sh.red[ww][piece][1], f, wsum);
-            const floatx4 ow = *reinterpret_cast<const floatx4 *>(&sh.red[ww][piece][4]);
+            wsum = __builtin_fmaf(sh.red[wv + ww][piece][1], f, wsum);
+            const floatx4 ow = *reinterpret_cast<const floatx4 *>(&sh.red[wv + ww][piece][4]);
 #pragma unroll
             for (int e = 0; e < 4; e++) {
                 osum[e] = __builtin_fmaf(ow[e], f, osum[e]);
@@ -1016,8 +1023,9 @@ __device__ inline void decode_body(const DecodeArgs &a, DecodeShared &sh) {
         const int q_begin = split * qps;
         const int q_end = (split + 1) * qps < total_quads ? (split + 1) * qps : total_quads;
         const int qw = 16 >> mg.sl_log;
-        const bool four = qps == 1 && a.nsplit > 64;  // all four waves on the one quad
-        if (q_begin >= q_end || (!four && q_begin + w * qw >= q_end)) {
+        // waves per quad when the slice is one or two quads of many splits (else a wave works alone)
+        const int wpq = (qps == 1 && a.nsplit > 64) ? 4 : (qps == 2 && a.nsplit > 32) ? 2 : 0;
+        if (q_begin >= q_end || (wpq == 0 && q_begin + w * qw >= q_end) || (wpq == 2 && q_begin + w / 2 >= q_end)) {
             return;
         }
         const unsigned long long t0 = wall_clock64();
@@ -1036,10 +1044,11 @@ __device__ inline void decode_body(const DecodeArgs &a, DecodeShared &sh) {
             }
         }
         TS(6);
-        int failed = four ? merge_quad4(mg, sh, q_begin, w, lane, t0, limit, a.flags)
-                          : merge_quads(mg, q_begin, q_end, w, W, lane, t0, limit);
+        int failed = wpq == 4   ? merge_quad_shared<4>(mg, sh, q_begin, q_end, w, lane, t0, limit, a.flags)
+                     : wpq == 2 ? merge_quad_shared<2>(mg, sh, q_begin, q_end, w, lane, t0, limit, a.flags)
+                                : merge_quads(mg, q_begin, q_end, w, W, lane, t0, limit);
         TS(7);
-        if (failed && (!four || w == 0)) {
+        if (failed && (wpq == 0 || w % wpq == 0)) {
             // Flag the slice (its own word, then the group's), then look once more, on its own and at
             // the whole slice.  (The look starts after the flags are known to be in place.)
             if (lane == 0) {
@@ -1131,8 +1140,8 @@ __global__ __launch_bounds__(kBlock) void decode_kernel(DecodeArgs a) {
         sh.p_ready = 0;
         sh.p_done = 0;
         sh.stored = 0;
-        sh.red_ready = 0;
-        sh.red_fail = 0;
+        sh.red_ready[0] = sh.red_ready[1] = 0;
+        sh.red_fail[0] = sh.red_fail[1] = 0;
     }
     __syncthreads();
     switch (a.rope.pairs > 0 ? a.rope.type : GLM_ATTN_ROPE_DISABLED) {

@@ -321,7 +321,7 @@ def test_decode_merge_geometries(H, h, kvh, max_length, n_past):
     p.close()
 
 
-@pytest.mark.parametrize("n_past", [200, 3000, 8191])
+@pytest.mark.parametrize("n_past", [200, 3000, 4095, 8191])
 def test_decode_slow_path_geometries(H, n_past):
     p = H.Pair(max_length=8192)
     p.ctx.set_spin_limit_us(0)
