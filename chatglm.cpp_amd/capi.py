@@ -152,7 +152,7 @@ DECODE_STAMPS = {
               (1, "queries in LDS (and the new key)"), (2, "maxes of the last round left"),
               (3, "probabilities of the last round left"), (6, "first look at the others' lines"),
               (13, "polling entered (last pass)"), (15, "last poll's loads back"), (12, "all lines in (last pass)"),
-              (4, "folded within the wave"), (11, "slice folded"), (7, "slice written")],
+              (11, "quads folded and written (last block)"), (7, "slice done")],
     "output": [(10, "wave started"), (0, "V column loads issued"), (3, "probabilities seen"), (4, "second product done"),
                (5, "lines issued")],
 }

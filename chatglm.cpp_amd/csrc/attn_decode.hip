@@ -57,25 +57,14 @@ static_assert(kDecodePartFloats == kMaxGroupHeads * QUADS * 16, "line layout");
 typedef unsigned int uintx4 __attribute__((ext_vector_type(4)));
 
 // ---------------------------------------------------------------------------------------------------
-// Lines of a split partial.  A line is four 16-byte pieces; piece p holds the launch's stamp, four
-// values of O / sum cut to 22 bits (sign, exponent, 13 mantissa bits, rounded to nearest: 2^-14
-// relative on values that are averages of V) and byte p of the fp32 base-2 log-sum-exp
-// max * log2(e) + log2(sum) of the (split, head).  A 16-byte store is performed as one, so a piece that shows the stamp is complete:
-// the data is its own ready flag.
-__device__ inline unsigned int round22(float x) {
-    const unsigned int u = __float_as_uint(x);
-    return x != x ? ((u | 0x00400000u) >> 10) : ((u + 0x200u) >> 10);
-}
-__device__ inline uintx4 pack_piece(unsigned int stamp, floatx4 v, unsigned int lse_bits, int p) {
-    const unsigned int a = round22(v[0]), b = round22(v[1]), c = round22(v[2]), d = round22(v[3]);
-    const unsigned int lse_byte = (lse_bits >> (8 * p)) & 0xffu;
-    return uintx4{stamp, a | (b << 22), (b >> 10) | (c << 12), (c >> 20) | (d << 2) | (lse_byte << 24)};
-}
-__device__ inline floatx4 unpack_piece(uintx4 r) {
-    const unsigned int a = r[1] & 0x3fffffu, b = (r[1] >> 22) | ((r[2] & 0xfffu) << 10);
-    const unsigned int c = (r[2] >> 12) | ((r[3] & 3u) << 20), d = (r[3] >> 2) & 0x3fffffu;
-    return floatx4{__uint_as_float(a << 10), __uint_as_float(b << 10), __uint_as_float(c << 10),
-                   __uint_as_float(d << 10)};
+// Lines of a split partial.  A line is four 16-byte pieces; a piece holds the launch's stamp, the fp32
+// base-2 log-sum-exp max * log2(e) + log2(sum) of the (split, head) and four values of O / sum as fp16
+// (O / sum is an average of fp16 V values: it cannot overflow, and the rounding is 2^-12 relative on a
+// partial whose weight in the result is at most 1).  A 16-byte store is performed as one, so a piece that
+// shows the stamp is complete with everything needed to fold it: the data is its own ready flag.
+__device__ inline uintx4 pack_piece(unsigned int stamp, floatx4 v, unsigned int lse_bits) {
+    const half2v a = {(_Float16)v[0], (_Float16)v[1]}, b = {(_Float16)v[2], (_Float16)v[3]};
+    return uintx4{stamp, lse_bits, __builtin_bit_cast(unsigned int, a), __builtin_bit_cast(unsigned int, b)};
 }
 
 // Data that crosses workgroups inside one launch moves with relaxed device-scope accesses: they are
@@ -322,11 +311,14 @@ __device__ inline half8 finish_q_part(const QPart &r, int d0, float scale, bool 
 }
 
 // ---------------------------------------------------------------------------------------------------
-// Merge across workgroups: fold the lines of all splits for quads [q_begin, q_end) of KV group g.
-// Quads are dealt out to the calling waves (wave `wi` of `nw`), `qw` of them at a time per wave: lane
-// (qslot, s, piece) takes piece `piece` of the lines of splits s, s + SL, ... of its quad.
+// Merge across workgroups: fold the lines of all splits for quads [q_begin, q_end) of KV group g (a quad
+// is 16 output dims of one head, index head * QUADS + quad).  A wave works alone on its quads, no LDS:
+// lane (s, quad slot, piece) takes piece `piece` of the lines of splits s, s + SL, ... of its quad, all
+// lines of a block of quads are loaded at once, and the split lanes of a quad are summed with cross-lane
+// operations.
 struct MergeGeom {
-    int nsplit, G, sl_log;  // SL = 1 << sl_log lanes per (quad, piece)
+    int nsplit, sl_log;  // SL = 1 << sl_log lanes per (quad, piece)
+    int nl;              // lines per lane and quad: ceil(nsplit / SL)
     unsigned int stamp32;
     const float *part_g;    // lines of the group: [16 heads][QUADS][nsplit][16 floats], a slice's lines side by side
     float *out_g;           // [G][D]
@@ -357,28 +349,35 @@ __device__ inline float reduce_splits(float x, int sl_log, F op) {
     return x;
 }
 
-// Polls lines `first + it * step` (it = 0 .. N - 1, those below nsplit) of one (quad, piece) until all have
-// arrived, then folds them into the lane's (max, sum, O) in the order of their index: the result does not
-// depend on the order in which the lines showed up.  A line counts when all four of its pieces carry the
-// stamp (its log-sum-exp is spread over them).  Returns 1 when the wait ran out.
+// (max, sum of weights, weighted O) of the lines a lane has folded, the weights relative to the max
 struct Fold {
     float m, w;
     floatx4 o;
 };
-template <int N>
-__device__ inline int poll_lines_n(const float *base, int first, int step, int nsplit, bool valid, unsigned int stamp32,
-                                   int piece, unsigned long long t0, unsigned long long limit, Fold &acc) {
+
+// One block of the merge: lines k0 .. k0 + NLP - 1 (line k is split k * SL + s) of the PC quads q[], all
+// loaded at once and polled until every one carries the stamp, then folded into acc[] in the order of their
+// index: the result does not depend on the order in which the lines showed up.  FIRST: acc[] is empty.
+// Returns 1 when the wait ran out.
+template <int NLP, int PC, bool FIRST>
+__device__ inline int poll_block(const MergeGeom &mg, const int (&q)[PC], const bool (&qvalid)[PC], int k0, int s,
+                                 int piece, unsigned long long t0, unsigned long long limit, Fold (&acc)[PC]) {
+    constexpr int N = NLP * PC;
     uintx4 r[N];
     const float *p[N];
     bool need[N];
     unsigned long long pending[N];
 #pragma unroll
-    for (int it = 0; it < N; it++) {
-        const int sp = first + it * step;
-        r[it] = uintx4{0u, 0u, 0u, 0u};
-        need[it] = valid && sp < nsplit;
-        p[it] = base + (sp < nsplit ? sp : 0) * 16;
-        pending[it] = __ballot(need[it]);
+    for (int pp = 0; pp < PC; pp++) {
+#pragma unroll
+        for (int k = 0; k < NLP; k++) {
+            const int i = pp * NLP + k;
+            const int sp = ((k0 + k) << mg.sl_log) + s;
+            r[i] = uintx4{0u, 0u, 0u, 0u};
+            need[i] = qvalid[pp] && sp < mg.nsplit;
+            p[i] = mg.part_g + ((int64_t)q[pp] * mg.nsplit + (sp < mg.nsplit ? sp : 0)) * 16 + piece * 4;
+            pending[i] = __ballot(need[i]);
+        }
     }
     TS(13);
     while (true) {
@@ -388,14 +387,10 @@ __device__ inline int poll_lines_n(const float *base, int first, int step, int n
         TS(15);
         unsigned long long any = 0ull;
 #pragma unroll
-        for (int it = 0; it < N; it++) {
-            if (pending[it] != 0ull) {
-                // all four pieces of a line: and over the quad of lanes
-                int ok = !need[it] || r[it][0] == stamp32;
-                ok &= __builtin_amdgcn_update_dpp(0, ok, 0xB1, 0xf, 0xf, true);  // quad_perm [1,0,3,2]
-                ok &= __builtin_amdgcn_update_dpp(0, ok, 0x4E, 0xf, 0xf, true);  // quad_perm [2,3,0,1]
-                pending[it] = __ballot(!ok);
-                any |= pending[it];
+        for (int i = 0; i < N; i++) {
+            if (pending[i] != 0ull) {
+                pending[i] = __ballot(need[i] && r[i][0] != mg.stamp32);
+                any |= pending[i];
             }
         }
         if (any == 0ull) {
@@ -407,50 +402,45 @@ __device__ inline int poll_lines_n(const float *base, int first, int step, int n
         __builtin_amdgcn_s_sleep(1);
     }
     TS(12);
-    // the base-2 log-sum-exp of each line from the bytes in its four pieces, and the new max
-    float lse[N];
-    float m_new = acc.m;
 #pragma unroll
-    for (int it = 0; it < N; it++) {
-        int bits = (int)(r[it][3] >> 24) << (8 * piece);
-        bits |= __builtin_amdgcn_update_dpp(0, bits, 0xB1, 0xf, 0xf, true);
-        bits |= __builtin_amdgcn_update_dpp(0, bits, 0x4E, 0xf, 0xf, true);
-        lse[it] = need[it] ? __int_as_float(bits) : -INFINITY;
-        m_new = fmaxf(m_new, lse[it]);
-    }
-    if (m_new != -INFINITY) {
-        const float sc = __builtin_amdgcn_exp2f(acc.m - m_new);  // exp2(-inf) = 0 for the first lines
-        acc.w *= sc;
-        acc.o *= sc;
-        acc.m = m_new;
+    for (int pp = 0; pp < PC; pp++) {
+        float lse[NLP];
+        float m_new = FIRST ? -INFINITY : acc[pp].m;
 #pragma unroll
-        for (int it = 0; it < N; it++) {
-            const float wgt = __builtin_amdgcn_exp2f(lse[it] - m_new);  // 0 for lines that are not there
-            const floatx4 v = unpack_piece(r[it]);
-            acc.w += wgt;
-#pragma unroll
-            for (int e = 0; e < 4; e++) {
-                acc.o[e] = __builtin_fmaf(wgt, v[e], acc.o[e]);
-            }
+        for (int k = 0; k < NLP; k++) {
+            lse[k] = need[pp * NLP + k] ? __uint_as_float(r[pp * NLP + k][1]) : -INFINITY;
+            m_new = fmaxf(m_new, lse[k]);
         }
+        const float m_ref = (m_new == -INFINITY) ? 0.f : m_new;  // nothing to fold: every weight below is 0
+        Fold f;
+        f.m = m_new;
+        if (FIRST) {
+            f.w = 0.f;
+            f.o = floatx4{0.f, 0.f, 0.f, 0.f};
+        } else {
+            const float sc = __builtin_amdgcn_exp2f(acc[pp].m - m_ref);  // exp2(-inf) = 0
+            f.w = acc[pp].w * sc;
+            f.o = acc[pp].o * sc;
+        }
+#pragma unroll
+        for (int k = 0; k < NLP; k++) {
+            const uintx4 rr = r[pp * NLP + k];
+            const float wgt = __builtin_amdgcn_exp2f(lse[k] - m_ref);  // 0 for lines that are not there
+            // (copies first: a bit cast straight from a vector element reads the vector's first element)
+            const unsigned int u0 = rr[2], u1 = rr[3];
+            const half2v h0 = __builtin_bit_cast(half2v, u0), h1 = __builtin_bit_cast(half2v, u1);
+            f.w += wgt;
+            f.o[0] = __builtin_fmaf(wgt, (float)h0[0], f.o[0]);
+            f.o[1] = __builtin_fmaf(wgt, (float)h0[1], f.o[1]);
+            f.o[2] = __builtin_fmaf(wgt, (float)h1[0], f.o[2]);
+            f.o[3] = __builtin_fmaf(wgt, (float)h1[1], f.o[3]);
+        }
+        acc[pp] = f;
     }
     return 0;
 }
 
-// b0: the first split of the pass (first = b0 + the lane's split slot).  The code that runs is the one for the
-// number of lines the pass really has per lane: at 2.3 ns a vector instruction, folding lines that are not
-// there costs as much as folding lines that are.
-__device__ inline int poll_lines(const float *base, int b0, int first, int step, int nsplit, bool valid,
-                                 unsigned int stamp32, int piece, unsigned long long t0, unsigned long long limit,
-                                 Fold &acc) {
-    const int n = (nsplit - b0 + step - 1) / step;  // the same in every lane
-    if (n <= 1) return poll_lines_n<1>(base, first, step, nsplit, valid, stamp32, piece, t0, limit, acc);
-    if (n <= 2) return poll_lines_n<2>(base, first, step, nsplit, valid, stamp32, piece, t0, limit, acc);
-    if (n <= 4) return poll_lines_n<4>(base, first, step, nsplit, valid, stamp32, piece, t0, limit, acc);
-    return poll_lines_n<8>(base, first, step, nsplit, valid, stamp32, piece, t0, limit, acc);
-}
-
-// What ends a slice: the (max, sum, O) of all lanes of a piece merged, normalised and stored.
+// What ends a quad: the (max, sum, O) of all lanes of a piece merged.
 __device__ inline void reduce_fold(Fold &acc, int sl_log) {
     const float m_all = reduce_splits(acc.m, sl_log, [](float x, float y) { return fmaxf(x, y); });
     const float f = (acc.m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(acc.m - m_all);
@@ -463,40 +453,63 @@ __device__ inline void reduce_fold(Fold &acc, int sl_log) {
     }
 }
 
-// Merges quads [q_begin, q_end) of KV group g, dealt out to the calling waves (wave `wi` of `nw`), `qw`
-// of them at a time per wave: lane (s, quad of the pass, piece) takes piece `piece` of the lines of
-// splits s, s + SL, ... of its quad.  Returns 0 when every quad was written, 1 when the wait ran out
-// (nothing is written for that pass).  Whoever completes quad 0 has seen a line of every workgroup of
-// the group: all of them have read the launch count by then, and it moves on.
-__device__ inline int merge_quads(const MergeGeom &mg, int q_begin, int q_end, int wi, int nw, int lane,
-                                  unsigned long long t0, unsigned long long limit) {
-    // s in the upper bits of the lane index, where reductions are cheap
-    const int SL = 1 << mg.sl_log, qw = 16 >> mg.sl_log;
+// The quads of the calling wave (wave `wi` of `nw`), PC passes of its QW quad slots at a time, NLP lines per lane
+// and block.
+template <int NLP, int PC>
+__device__ inline int merge_passes(const MergeGeom &mg, int q_begin, int q_end, int wi, int nw, int lane,
+                                   unsigned long long t0, unsigned long long limit) {
+    const int qw = 16 >> mg.sl_log;
     const int piece = lane & 3, qslot = (lane >> 2) & (qw - 1), s = lane >> (6 - mg.sl_log);
-    for (int q0 = q_begin + wi * qw; q0 < q_end; q0 += nw * qw) {
-        const int q = q0 + qslot;
-        const bool valid = q < q_end;
-        const int qc = valid ? q : q_end - 1;
-        const int hd = qc / QUADS, quad = qc - hd * QUADS;
-        const float *base = mg.part_g + ((int64_t)(hd * QUADS + quad) * mg.nsplit * 4 + piece) * 4;
-        Fold acc = {-INFINITY, 0.f, floatx4{0.f, 0.f, 0.f, 0.f}};
-        for (int b0 = 0; b0 < mg.nsplit; b0 += 8 * SL) {
-            if (poll_lines(base, b0, b0 + s, SL, mg.nsplit, valid, mg.stamp32, piece, t0, limit, acc)) {
+    for (int q0 = q_begin + wi * qw; q0 < q_end; q0 += PC * nw * qw) {
+        int q[PC];
+        bool qvalid[PC];
+        Fold acc[PC];
+#pragma unroll
+        for (int pp = 0; pp < PC; pp++) {
+            const int qq = q0 + pp * nw * qw + qslot;
+            qvalid[pp] = qq < q_end;
+            q[pp] = qvalid[pp] ? qq : q_end - 1;
+        }
+        if (poll_block<NLP, PC, true>(mg, q, qvalid, 0, s, piece, t0, limit, acc)) {
+            return 1;
+        }
+        for (int k0 = NLP; k0 < mg.nl; k0 += NLP) {
+            if (poll_block<NLP, PC, false>(mg, q, qvalid, k0, s, piece, t0, limit, acc)) {
                 return 1;
             }
         }
-        reduce_fold(acc, mg.sl_log);
+#pragma unroll
+        for (int pp = 0; pp < PC; pp++) {
+            if (q0 + pp * nw * qw < q_end) {  // the same in every lane
+                reduce_fold(acc[pp], mg.sl_log);
+                if (qvalid[pp] && s == 0) {
+                    // (1 / sum to one ulp, then a product: the values were rounded to fp16 on their way here)
+                    *reinterpret_cast<floatx4 *>(mg.out_g + q[pp] * 16 + piece * 4) =
+                        acc[pp].o * __builtin_amdgcn_rcpf(acc[pp].w);
+                }
+            }
+        }
         TS(11);
-        if (valid && s == 0) {
-            // (1 / sum to one ulp, then a product: the values were cut to 22 bits on their way here)
-            *reinterpret_cast<floatx4 *>(mg.out_g + hd * D + quad * 16 + piece * 4) =
-                acc.o * __builtin_amdgcn_rcpf(acc.w);
-        }
-        if (q0 == 0 && lane == 0) {
-            __hip_atomic_store(mg.gen_word, mg.gen_next, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
     }
     return 0;
+}
+
+// Merges quads [q_begin, q_end) of KV group g, dealt out to the calling waves (wave `wi` of `nw`).  Returns 0 when
+// every quad was written, 1 when the wait ran out (the quads of the block that was being waited for, and the wave's
+// later ones, are not written).  Whoever completes a quad has seen a line of every workgroup of the group: all of
+// them have read the launch count by then, and it may move on (`bump`: this caller is one of those that say so).
+__device__ inline int merge_quads(const MergeGeom &mg, int q_begin, int q_end, int wi, int nw, int lane,
+                                  unsigned long long t0, unsigned long long limit, bool bump) {
+    // the code that runs is the one for the number of lines a lane really has: at 2.3 ns a vector instruction,
+    // folding lines that are not there costs as much as folding lines that are
+    const int failed = mg.nl <= 1   ? merge_passes<1, 4>(mg, q_begin, q_end, wi, nw, lane, t0, limit)
+                       : mg.nl <= 2 ? merge_passes<2, 2>(mg, q_begin, q_end, wi, nw, lane, t0, limit)
+                       : mg.nl <= 4 ? merge_passes<4, 1>(mg, q_begin, q_end, wi, nw, lane, t0, limit)
+                                    : merge_passes<8, 1>(mg, q_begin, q_end, wi, nw, lane, t0, limit);
+    if (!failed && bump && lane == 0) {
+        __hip_atomic_store(mg.gen_word, mg.gen_next, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    return failed;
 }
 
 // Before its first look at the lines of the others a wave waits 0.7 us plus 0.12 us per 4096 keys of the group
@@ -521,10 +534,6 @@ struct DecodeShared {
     int p_ready;        // score waves that have left their part of P, over all rounds
     int p_done;         // output waves that are through with P, over all rounds
     int stored;         // output waves whose line stores have been performed
-    // several score waves on one quad of the output: what each leaves for the first of them
-    float red[W][4][8];  // per wave and piece: max, sum, O[4]
-    int red_ready[2];    // per quad of the workgroup's slice (one, or two with two waves each)
-    int red_fail[2];
 };
 
 // A wave waits for waves of its own workgroup (all resident by construction) through a counter in LDS.
@@ -558,74 +567,6 @@ __device__ inline float sum_over_c(float x) {
     x = __uint_as_float(a[0]) + __uint_as_float(a[1]);
     auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
     return __uint_as_float(b[0]) + __uint_as_float(b[1]);
-}
-
-// Many splits and a slice of one or two quads: WPQ = 4 or 2 score waves work on a quad, 16 split lanes each, and
-// the first of them finishes it from what the others leave in LDS.  wv: the wave among the score waves; its quad is
-// q_begin + wv / WPQ (a wave whose quad lies beyond the slice has nothing to do).
-template <int WPQ>
-__device__ inline int merge_quad_shared(const MergeGeom &mg, DecodeShared &sh, int q_begin, int q_end, int wv, int lane,
-                                        unsigned long long t0, unsigned long long limit, uint32_t *flags) {
-    const int ql = wv / WPQ, sub = wv % WPQ;
-    const int q = q_begin + ql;
-    if (q >= q_end) {
-        return 0;
-    }
-    const int piece = lane & 3, s = sub * 16 + (lane >> 2);
-    const int hd = q / QUADS, quad = q - hd * QUADS;
-    const float *base = mg.part_g + ((int64_t)(hd * QUADS + quad) * mg.nsplit * 4 + piece) * 4;
-    Fold acc = {-INFINITY, 0.f, floatx4{0.f, 0.f, 0.f, 0.f}};
-    int failed = 0;
-    for (int b0 = 0; b0 < mg.nsplit && !failed; b0 += 8 * 16 * WPQ) {
-        failed = poll_lines(base, b0, b0 + s, 16 * WPQ, mg.nsplit, true, mg.stamp32, piece, t0, limit, acc);
-    }
-    reduce_fold(acc, 4);
-    TS(4);
-    if (lane < 4) {
-        float *dst = &sh.red[wv][piece][0];
-        dst[0] = acc.m;
-        dst[1] = acc.w;
-        *reinterpret_cast<floatx4 *>(dst + 4) = acc.o;
-        if (failed) {
-            sh.red_fail[ql] = 1;
-        }
-    }
-    lds_signal(&sh.red_ready[ql], lane);
-    if (sub != 0) {
-        return failed;
-    }
-    lds_wait_ge(&sh.red_ready[ql], WPQ, flags);
-    failed |= __hip_atomic_load(&sh.red_fail[ql], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-    if (failed) {
-        return 1;
-    }
-    if (lane < 4) {
-        float m_all = acc.m;
-#pragma unroll
-        for (int ww = 1; ww < WPQ; ww++) {
-            m_all = fmaxf(m_all, sh.red[wv + ww][piece][0]);
-        }
-        float f = (acc.m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(acc.m - m_all);
-        float wsum = acc.w * f;
-        floatx4 osum = acc.o * f;
-#pragma unroll
-        for (int ww = 1; ww < WPQ; ww++) {
-            const float mw = sh.red[wv + ww][piece][0];
-            f = (mw == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(mw - m_all);
-            wsum = __builtin_fmaf(sh.red[wv + ww][piece][1], f, wsum);
-            const floatx4 ow = *reinterpret_cast<const floatx4 *>(&sh.red[wv + ww][piece][4]);
-#pragma unroll
-            for (int e = 0; e < 4; e++) {
-                osum[e] = __builtin_fmaf(ow[e], f, osum[e]);
-            }
-        }
-        TS(11);
-        *reinterpret_cast<floatx4 *>(mg.out_g + hd * D + quad * 16 + piece * 4) = osum * __builtin_amdgcn_rcpf(wsum);
-    }
-    if (q == 0 && lane == 0) {
-        __hip_atomic_store(mg.gen_word, mg.gen_next, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    return 0;
 }
 
 // A slice that was left behind has been written after all: whoever takes the flag off takes it off the
@@ -984,15 +925,11 @@ __device__ inline void decode_body(const DecodeArgs &a, DecodeShared &sh) {
     auto resolve = [&]() {
         qps = (total_quads + a.nsplit - 1) / a.nsplit;
         mg.nsplit = a.nsplit;
-        mg.G = G;
         mg.sl_log = 0;
         while (mg.sl_log < 4 && (1 << mg.sl_log) < a.nsplit) {
             mg.sl_log++;
         }
-        // ... but no more split lanes than leave a wave room for its share of the slice's quads in one pass
-        while (mg.sl_log > 0 && (16 >> mg.sl_log) * W < qps) {
-            mg.sl_log--;
-        }
+        mg.nl = (a.nsplit + (1 << mg.sl_log) - 1) >> mg.sl_log;
         mg.part_g = a.part + (int64_t)g * a.nsplit * kDecodePartFloats;
         mg.out_g = a.out + (int64_t)g * G * D;
         mg.gen_word = &a.sync[g].gen;
@@ -1023,10 +960,8 @@ __device__ inline void decode_body(const DecodeArgs &a, DecodeShared &sh) {
         const int q_begin = split * qps;
         const int q_end = (split + 1) * qps < total_quads ? (split + 1) * qps : total_quads;
         const int qw = 16 >> mg.sl_log;
-        // waves per quad when the slice is one or two quads of many splits (else a wave works alone)
-        const int wpq = (qps == 1 && a.nsplit > 64) ? 4 : (qps == 2 && a.nsplit > 32) ? 2 : 0;
-        if (q_begin >= q_end || (wpq == 0 && q_begin + w * qw >= q_end) || (wpq == 2 && q_begin + w / 2 >= q_end)) {
-            return;
+        if (q_begin + w * qw >= q_end) {
+            return;  // fewer quads in the slice than the score waves take in one pass
         }
         const unsigned long long t0 = wall_clock64();
         const unsigned long long limit = (unsigned long long)a.spin_ticks;
@@ -1044,11 +979,10 @@ __device__ inline void decode_body(const DecodeArgs &a, DecodeShared &sh) {
             }
         }
         TS(6);
-        int failed = wpq == 4   ? merge_quad_shared<4>(mg, sh, q_begin, q_end, w, lane, t0, limit, a.flags)
-                     : wpq == 2 ? merge_quad_shared<2>(mg, sh, q_begin, q_end, w, lane, t0, limit, a.flags)
-                                : merge_quads(mg, q_begin, q_end, w, W, lane, t0, limit);
+        // (the first slices' first waves move the launch count on: any of them is enough)
+        const int failed = merge_quads(mg, q_begin, q_end, w, W, lane, t0, limit, split < 4 && w == 0);
         TS(7);
-        if (failed && (wpq == 0 || w % wpq == 0)) {
+        if (failed) {
             // Flag the slice (its own word, then the group's), then look once more, on its own and at
             // the whole slice.  (The look starts after the flags are known to be in place.)
             if (lane == 0) {
@@ -1060,7 +994,7 @@ __device__ inline void decode_body(const DecodeArgs &a, DecodeShared &sh) {
                 __hip_atomic_store(&sy->flagged, stamp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
             wait_vm();
-            if (!merge_quads(mg, q_begin, q_end, 0, 1, lane, wall_clock64(), 0ull)) {
+            if (!merge_quads(mg, q_begin, q_end, 0, 1, lane, wall_clock64(), 0ull, split < 4)) {
                 slice_redone(claim + split, stamp, &sy->lost, lane);
             }
         }
@@ -1095,7 +1029,7 @@ __device__ inline void decode_body(const DecodeArgs &a, DecodeShared &sh) {
 #pragma unroll
         for (int jb = 0; jb < 2; jb++) {
             st_dev4(pw + (int64_t)(j * QUADS + w * 2 + jb) * a.nsplit * 16 + c * 4,
-                    pack_piece(stamp32, o[jb] * inv, lse, c));
+                    pack_piece(stamp32, o[jb] * inv, lse));
         }
     }
     TS(5);
@@ -1123,8 +1057,10 @@ __device__ inline void decode_body(const DecodeArgs &a, DecodeShared &sh) {
             left &= left - 1;
             const int qb = sl * qps;
             const int qe = (sl + 1) * qps < total_quads ? (sl + 1) * qps : total_quads;
-            if (!merge_quads(mg, qb, qe, 0, 1, lane, wall_clock64(), sweep_limit)) {
+            if (!merge_quads(mg, qb, qe, 0, 1, lane, wall_clock64(), sweep_limit, sl < 4)) {
                 slice_redone(claim + sl, stamp, &sy->lost, lane);
+            } else if (lane == 0) {
+                atomicOr(a.flags, kFlagMergeIncomplete);  // even the long wait ran out: reported for good
             }
         }
     }
@@ -1140,8 +1076,6 @@ __global__ __launch_bounds__(kBlock) void decode_kernel(DecodeArgs a) {
         sh.p_ready = 0;
         sh.p_done = 0;
         sh.stored = 0;
-        sh.red_ready[0] = sh.red_ready[1] = 0;
-        sh.red_fail[0] = sh.red_fail[1] = 0;
     }
     __syncthreads();
     switch (a.rope.pairs > 0 ? a.rope.type : GLM_ATTN_ROPE_DISABLED) {
