@@ -63,17 +63,21 @@ def fill_cache_normal(torch, kv, seed):
 def read_ceilings(torch, pkg, kv, layer_halfs, stream, warmup, steps):
     """Kernels that only load, launched like the decode step: LAYERS launches back to back on one stream, each
     over another layer's 32 MiB of cache, timed with events on that stream."""
-    lib = pkg.lib()
+    lib = pkg.bench_lib()
     sink = torch.zeros(1, dtype=torch.float32, device=kv.device)
     sh = stream.cuda_stream
     layer_bytes = layer_halfs * 2
     base = kv.data_ptr()
 
-    def run(pattern, per_launch_bytes, launches, whole=False):
+    def run(pattern, per_launch_bytes, launches, whole=False, sweep=None):
         def step():
             for l in range(launches):
                 ptr = base if whole else base + l * layer_bytes
-                st = lib.glm_bench_read(pattern, ptr, MAX_LENGTH, KVH, per_launch_bytes, sink.data_ptr(), sh)
+                if sweep is None:
+                    st = lib.glm_bench_read(pattern, ptr, MAX_LENGTH, KVH, per_launch_bytes, sink.data_ptr(), sh)
+                else:
+                    st = lib.glm_bench_read_sweep(sweep[0], sweep[1], sweep[2], sweep[3], ptr, per_launch_bytes,
+                                                  sink.data_ptr(), sh)
                 if st != 0:
                     pkg.check(st, "glm_bench_read")
 
@@ -100,6 +104,25 @@ def read_ceilings(torch, pkg, kv, layer_halfs, stream, warmup, steps):
     out["linear_read_per_launch"] = run(pkg.BENCH_READ_LINEAR, layer_bytes, LAYERS)
     out["decode_pattern_read_per_launch"] = run(pkg.BENCH_READ_DECODE_PATTERN, layer_bytes, LAYERS)
     out["one_long_streaming_launch"] = run(pkg.BENCH_READ_STREAM, layer_bytes * LAYERS, 1, whole=True)
+    # The same 32 MiB per launch asked for in other ways: workgroups of 4, 8 or 16 waves, 8 to 32 loads of 16 bytes
+    # per lane in flight, cache policy bits, straight into LDS.  The best of them is the ceiling.
+    sweep = {}
+    policies = (("plain", pkg.BENCH_POLICY_PLAIN), ("nt", pkg.BENCH_POLICY_NT), ("sc1", pkg.BENCH_POLICY_SC1),
+                ("sc0_sc1_nt", pkg.BENCH_POLICY_SC0_SC1_NT))
+    shapes = ((8, 16), (4, 16), (4, 32), (16, 8), (8, 8), (4, 8), (16, 16))
+    for pname, pol in policies:
+        for waves, loads in shapes:
+            r = run(None, layer_bytes, LAYERS, sweep=(pol, waves, loads, 0))
+            sweep[f"{pname}, {layer_bytes // (waves * loads * 1024)} workgroups x {waves} waves x {loads} loads"] = r
+    for pname, pol in policies[:2]:
+        for waves, loads in ((8, 16), (4, 16), (4, 32)):
+            r = run(None, layer_bytes, LAYERS, sweep=(pol, waves, loads, 1))
+            sweep[f"{pname} into LDS, {layer_bytes // (waves * loads * 1024)} workgroups x {waves} waves x {loads} "
+                  "loads"] = r
+    best = min(sweep, key=lambda k: sweep[k]["us_per_launch"])
+    out["sweep"] = {k: {"us_per_launch": v["us_per_launch"], "frac_of_hbm_peak": v["frac_of_hbm_peak"]}
+                    for k, v in sweep.items()}
+    out["best_read_per_launch"] = dict(sweep[best], shape=best)
     return out
 
 
@@ -108,7 +131,7 @@ def mfma_ceilings(torch, pkg, stream):
     the clock to settle: what the matrix pipes give any kernel here, beside the prefill kernel's rate."""
     import ctypes
 
-    lib = pkg.lib()
+    lib = pkg.bench_lib()
     dev = torch.device("cuda:0")
     operands = (torch.rand(1 << 16, device=dev, dtype=torch.float32) - 0.5).to(torch.float16)  # 128 KiB
     sink = torch.zeros(1, dtype=torch.float32, device=dev)

@@ -19,7 +19,7 @@ MASK_RULE_REFERENCE, MASK_RULE_CAUSAL_OFFSET = 0, 1
 # every symbol include/glm_attn.h declares
 SYMBOLS = [
     "glm_attn_default_desc", "glm_attn_kv_bytes", "glm_attn_create", "glm_attn_destroy", "glm_attn_cache_ptrs",
-    "glm_attn_forward", "glm_attn_rope_append", "glm_attn_decode", "glm_attn_decode_static", "glm_attn_prefill",
+    "glm_attn_forward", "glm_attn_rope_append", "glm_attn_attend", "glm_attn_decode", "glm_attn_decode_static", "glm_attn_prefill",
     "glm_attn_load_prefix_cache", "glm_attn_position_ids_glm2", "glm_attn_position_ids_glm",
     "glm_attn_attention_mask_glm", "glm_attn_scale_add", "glm_attn_device_flags", "glm_attn_set_spin_limit_us", "glm_attn_last_hip_error", "glm_attn_strerror",
     "glm_attn_version",
@@ -40,7 +40,8 @@ MODEL_FILE_SYMBOLS = [
     "glm_model_file_data", "glm_model_file_tensor_count", "glm_model_file_tensor", "glm_model_file_find",
     "glm_model_file_upload",
 ]
-BENCH_SYMBOLS = ["glm_bench_mfma", "glm_bench_read"]
+BENCH_SYMBOLS = ["glm_bench_mfma", "glm_bench_read", "glm_bench_read_sweep"]
+BENCH_POLICY_PLAIN, BENCH_POLICY_NT, BENCH_POLICY_SC1, BENCH_POLICY_SC0_SC1_NT = 0, 1, 2, 3
 BENCH_MFMA_32X32X16, BENCH_MFMA_16X16X32, BENCH_MFMA_32X32X16_MIX, BENCH_MFMA_16X16X32_MIX = 0, 1, 2, 3
 BENCH_READ_LINEAR, BENCH_READ_DECODE_PATTERN, BENCH_READ_STREAM, BENCH_EMPTY = 0, 1, 2, 3
 MODEL_F32, MODEL_F16, MODEL_Q4_0, MODEL_Q4_1, MODEL_Q5_0, MODEL_Q5_1, MODEL_Q8_0 = 0, 1, 2, 3, 6, 7, 8
@@ -207,6 +208,31 @@ def summarise_timeline(t, stamps, rows):
     return out
 
 
+BENCH_LIB_PATH = os.path.join(_PKG, "libglm_bench.so")
+_bench_lib = None
+
+
+def bench_lib():
+    """The measurement aids of include/glm_bench.h (libglm_bench.so): read kernels and loops of matrix
+    instructions that bench.py --ceiling times beside the kernels of the path.  No part of the drop-in library."""
+    global _bench_lib
+    if _bench_lib is not None:
+        return _bench_lib
+    if not os.path.exists(BENCH_LIB_PATH):
+        raise RuntimeError(f"{BENCH_LIB_PATH} is missing: build it with __graft_entry__.build()")
+    c = ctypes
+    P = c.c_void_p
+    L = c.CDLL(BENCH_LIB_PATH)
+    L.glm_bench_read.argtypes = [c.c_int, P, c.c_int32, c.c_int32, c.c_size_t, P, P]
+    L.glm_bench_read.restype = c.c_int
+    L.glm_bench_read_sweep.argtypes = [c.c_int, c.c_int32, c.c_int32, c.c_int32, P, c.c_size_t, P, P]
+    L.glm_bench_read_sweep.restype = c.c_int
+    L.glm_bench_mfma.argtypes = [c.c_int, P, c.c_size_t, c.c_int32, P, P, c.POINTER(c.c_double)]
+    L.glm_bench_mfma.restype = c.c_int
+    _bench_lib = L
+    return L
+
+
 def lib():
     global _lib
     if _lib is not None:
@@ -231,6 +257,8 @@ def lib():
     L.glm_attn_forward.restype = c.c_int
     L.glm_attn_rope_append.argtypes = [P, c.c_int32, P, c.c_int64, P, c.c_int32, c.c_int32, P]
     L.glm_attn_rope_append.restype = c.c_int
+    L.glm_attn_attend.argtypes = [P, c.c_int32, P, c.c_int32, c.c_int32, P, P]
+    L.glm_attn_attend.restype = c.c_int
     L.glm_attn_decode.argtypes = [P, c.c_int32, P, P, P, c.c_int32, P, P]
     L.glm_attn_decode.restype = c.c_int
     L.glm_attn_decode_static.argtypes = [P, c.c_int32, P, P, P, c.c_int32, P, P]
@@ -283,10 +311,6 @@ def lib():
     L.glm_block_gated_activation.restype = c.c_int
     L.glm_block_embedding.argtypes = [P, c.c_int32, c.c_int64, c.c_int32, P, c.c_int32, P, P]
     L.glm_block_embedding.restype = c.c_int
-    L.glm_bench_read.argtypes = [c.c_int, P, c.c_int32, c.c_int32, c.c_size_t, P, P]
-    L.glm_bench_read.restype = c.c_int
-    L.glm_bench_mfma.argtypes = [c.c_int, P, c.c_size_t, c.c_int32, P, P, c.POINTER(c.c_double)]
-    L.glm_bench_mfma.restype = c.c_int
     L.glm_model_file_open.argtypes = [c.c_char_p, c.POINTER(P)]
     L.glm_model_file_open.restype = c.c_int
     L.glm_model_file_close.argtypes = [P]
@@ -375,6 +399,9 @@ class Context:
     def rope_append(self, layer, qkv_ptr, position_ids_ptr, qlen, n_past, qkv_row_stride=0, stream=None):
         return lib().glm_attn_rope_append(self.handle, layer, qkv_ptr, qkv_row_stride, position_ids_ptr, qlen, n_past,
                                           stream)
+
+    def attend(self, layer, qlen, n_past, out_ptr, attention_mask_ptr=None, stream=None):
+        return lib().glm_attn_attend(self.handle, layer, attention_mask_ptr, qlen, n_past, out_ptr, stream)
 
     def decode(self, layer, qkv_ptr, n_past, out_ptr, position_ids_ptr=None, position_ids_host=None, stream=None):
         hp = None

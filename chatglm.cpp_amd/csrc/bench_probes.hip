@@ -1,7 +1,8 @@
 // Read kernels that do nothing but load: what this GPU gives a launch shaped like the decode kernel's
 // (one workgroup per CU, every load of the launch issued up front), with the arithmetic, the exchange
 // between workgroups and the output taken away; and loops of matrix instructions: what the matrix pipes give
-// the prefill kernel.  bench.py --ceiling times them; they are no part of the attention path.
+// the prefill kernel.  bench.py --ceiling times them; they are no part of the attention path and are built
+// into a library of their own (libglm_bench.so).
 #include "glm_attn_internal.h"
 #include "glm_bench.h"
 
@@ -100,6 +101,118 @@ __global__ void empty_kernel(float *sink, int never) {
     if (never == 12345 && threadIdx.x == 77) {
         sink[0] = 1.f;
     }
+}
+
+// ---- the same bytes asked for in other ways: what shape of launch, how many loads in flight per wave and
+// which cache policy bits read fastest.  One launch reads `bytes` contiguous bytes with bytes / (W * NL KiB)
+// workgroups of W waves, every lane NL loads of 16 bytes, all issued before the one wait.
+typedef unsigned int uintx4 __attribute__((ext_vector_type(4)));
+
+// POL 0: plain, 1: nt (non-temporal), 2: sc1, 3: sc0 sc1 nt.  The result register of every load is used after
+// the wait in the kernel, so it stays reserved while the load is on its way.
+template <int POL>
+__device__ inline void ld_policy(uintx4 &r, const void *p) {
+    if (POL == 0) asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(r) : "v"(p) : "memory");
+    if (POL == 1) asm volatile("global_load_dwordx4 %0, %1, off nt" : "=v"(r) : "v"(p) : "memory");
+    if (POL == 2) asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(r) : "v"(p) : "memory");
+    if (POL == 3) asm volatile("global_load_dwordx4 %0, %1, off sc0 sc1 nt" : "=v"(r) : "v"(p) : "memory");
+}
+
+template <int POL, int W, int NL>
+__global__ __launch_bounds__(W * 64) void sweep_kernel(const char *base, float *sink) {
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    uintx4 r[NL];
+    const char *p = base + (size_t)blockIdx.x * (W * NL * 1024) + (size_t)w * (NL * 1024) + lane * 16;
+#pragma unroll
+    for (int i = 0; i < NL; i++) {
+        ld_policy<POL>(r[i], p + i * 1024);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    unsigned int acc = 0;
+#pragma unroll
+    for (int i = 0; i < NL; i++) {
+        asm volatile("" : "+v"(r[i]));
+        acc ^= r[i][0] ^ r[i][1] ^ r[i][2] ^ r[i][3];
+    }
+    if (acc == 0x12345679u) {
+        sink[0] = 1.f;  // practically never: keeps the loads alive
+    }
+}
+
+// The same through LDS: global_load_lds_dwordx4 drops the 64 lanes' 16 bytes at consecutive LDS addresses and
+// needs no registers.  W * NL KiB of LDS per workgroup.  POL 0: plain, 1: nt.
+template <int POL, int W, int NL>
+__global__ __launch_bounds__(W * 64) void sweep_lds_kernel(const char *base, float *sink) {
+    extern __shared__ char lds[];
+    const int lane = threadIdx.x & 63;
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const char *p = base + (size_t)blockIdx.x * (W * NL * 1024) + (size_t)w * (NL * 1024);
+    const uint32_t lds0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)lds) + w * NL * 1024;
+#pragma unroll
+    for (int i = 0; i < NL; i++) {
+        const uint32_t dst = lds0 + i * 1024;
+        const uint32_t off = i * 1024 + lane * 16;
+        if (POL == 0) {
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                         : : "s"(dst), "v"(off), "s"(p) : "memory");
+        } else {
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt"
+                         : : "s"(dst), "v"(off), "s"(p) : "memory");
+        }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    const unsigned int acc = *reinterpret_cast<unsigned int *>(lds + threadIdx.x * 4);
+    if (acc == 0x12345679u) {
+        sink[0] = 1.f;  // practically never
+    }
+}
+
+template <int POL, int W, int NL>
+hipError_t launch_sweep(const char *base, size_t bytes, float *sink, hipStream_t st) {
+    hipLaunchKernelGGL((sweep_kernel<POL, W, NL>), dim3((unsigned int)(bytes / ((size_t)W * NL * 1024))), dim3(W * 64), 0,
+                       st, base, sink);
+    return hipGetLastError();
+}
+template <int POL, int W, int NL>
+hipError_t launch_sweep_lds(const char *base, size_t bytes, float *sink, hipStream_t st) {
+    constexpr int kLds = W * NL * 1024;
+    static bool raised = false;  // more than 64 KiB of LDS wants the limit raised once
+    if (!raised) {
+        hipError_t e = hipFuncSetAttribute((const void *)sweep_lds_kernel<POL, W, NL>,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
+        if (e != hipSuccess) return e;
+        raised = true;
+    }
+    hipLaunchKernelGGL((sweep_lds_kernel<POL, W, NL>), dim3((unsigned int)(bytes / ((size_t)W * NL * 1024))), dim3(W * 64),
+                       kLds, st, base, sink);
+    return hipGetLastError();
+}
+template <int POL>
+hipError_t launch_sweep_shape(int waves, int loads, int through_lds, const char *base, size_t bytes, float *sink,
+                              hipStream_t st, bool *known) {
+    *known = true;
+    if (through_lds) {
+        constexpr int P2 = POL > 1 ? 0 : POL;
+        if (POL > 1) {
+            *known = false;
+            return hipSuccess;
+        }
+        if (waves == 8 && loads == 16) return launch_sweep_lds<P2, 8, 16>(base, bytes, sink, st);
+        if (waves == 4 && loads == 16) return launch_sweep_lds<P2, 4, 16>(base, bytes, sink, st);
+        if (waves == 4 && loads == 32) return launch_sweep_lds<P2, 4, 32>(base, bytes, sink, st);
+        *known = false;
+        return hipSuccess;
+    }
+    if (waves == 8 && loads == 16) return launch_sweep<POL, 8, 16>(base, bytes, sink, st);
+    if (waves == 4 && loads == 16) return launch_sweep<POL, 4, 16>(base, bytes, sink, st);
+    if (waves == 4 && loads == 32) return launch_sweep<POL, 4, 32>(base, bytes, sink, st);
+    if (waves == 16 && loads == 8) return launch_sweep<POL, 16, 8>(base, bytes, sink, st);
+    if (waves == 8 && loads == 8) return launch_sweep<POL, 8, 8>(base, bytes, sink, st);
+    if (waves == 4 && loads == 8) return launch_sweep<POL, 4, 8>(base, bytes, sink, st);
+    if (waves == 16 && loads == 16) return launch_sweep<POL, 16, 16>(base, bytes, sink, st);
+    *known = false;
+    return hipSuccess;
 }
 
 }  // namespace
@@ -234,6 +347,35 @@ extern "C" int glm_bench_mfma(int pattern, const void *operands, size_t operand_
         *flops = (double)grid.x * 4.0 * iters * 8.0 * 4.0 * 32.0 * 32.0 * 16.0 * 2.0;
     }
     return hipGetLastError() == hipSuccess ? GLM_ATTN_OK : GLM_ATTN_EHIP;
+}
+
+extern "C" int glm_bench_read_sweep(int policy, int32_t waves, int32_t loads, int32_t through_lds, const void *base,
+                                    size_t bytes, float *sink, void *stream) {
+    if (!base || !sink || waves <= 0 || loads <= 0) return GLM_ATTN_EINVAL;
+    const size_t per_wg = (size_t)waves * loads * 1024;
+    if (bytes < per_wg || bytes % per_wg != 0 || bytes / per_wg > 0x7fffffffu) return GLM_ATTN_EINVAL;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const char *b = static_cast<const char *>(base);
+    bool known = false;
+    hipError_t e = hipSuccess;
+    switch (policy) {
+    case GLM_BENCH_POLICY_PLAIN:
+        e = launch_sweep_shape<0>(waves, loads, through_lds, b, bytes, sink, st, &known);
+        break;
+    case GLM_BENCH_POLICY_NT:
+        e = launch_sweep_shape<1>(waves, loads, through_lds, b, bytes, sink, st, &known);
+        break;
+    case GLM_BENCH_POLICY_SC1:
+        e = launch_sweep_shape<2>(waves, loads, through_lds, b, bytes, sink, st, &known);
+        break;
+    case GLM_BENCH_POLICY_SC0_SC1_NT:
+        e = launch_sweep_shape<3>(waves, loads, through_lds, b, bytes, sink, st, &known);
+        break;
+    default:
+        return GLM_ATTN_EINVAL;
+    }
+    if (!known) return GLM_ATTN_EUNSUPPORTED;
+    return e == hipSuccess ? GLM_ATTN_OK : GLM_ATTN_EHIP;
 }
 
 extern "C" int glm_bench_read(int pattern, const void *base, int32_t cache_rows, int32_t kv_heads, size_t bytes,

@@ -530,6 +530,25 @@ int glm_attn_prefill(glm_attn_ctx *ctx, int32_t layer, const float *qkv, int64_t
     return GLM_ATTN_OK;
 }
 
+int glm_attn_attend(glm_attn_ctx *ctx, int32_t layer, const float *attention_mask, int32_t qlen, int32_t n_past,
+                    float *out, void *stream) {
+    int rc = check_call(ctx, layer, qlen, n_past);
+    if (rc != GLM_ATTN_OK) return rc;
+    if (!out) return GLM_ATTN_EINVAL;
+    int causal;
+    const float *mask;
+    rc = resolve_mask(ctx, n_past, attention_mask, &causal, &mask);
+    if (rc != GLM_ATTN_OK) return rc;
+    DeviceGuard guard(ctx->desc.device);
+    AttendArgs aa = make_attend(ctx, layer, qlen, n_past, causal, mask, out);
+    if (ctx->fast && aligned16(out)) {
+        HIP_TRY(ctx, launch_prefill(aa, ctx->num_cus, (hipStream_t)stream));
+    } else {
+        HIP_TRY(ctx, launch_attend_generic(aa, (hipStream_t)stream));
+    }
+    return GLM_ATTN_OK;
+}
+
 int glm_attn_forward(glm_attn_ctx *ctx, int32_t layer, const float *qkv, int64_t qkv_row_stride,
                      const float *attention_mask, const int32_t *position_ids, const int32_t *position_ids_host,
                      int32_t qlen, int32_t n_past, float *out, void *stream) {
@@ -605,6 +624,16 @@ int glm_attn_device_flags(glm_attn_ctx *ctx, uint32_t *flags) {
     HIP_TRY(ctx, hipMemcpy(sync.data(), ctx->sync, sync.size() * sizeof(DecodeGroupSync), hipMemcpyDeviceToHost));
     for (const DecodeGroupSync &g : sync) {
         if (g.lost != 0) *flags |= kFlagMergeIncomplete;
+    }
+    // ... and the same count of the device's static exchange memory (glm_attn_decode_static), which every
+    // context on the device shares: a slice lost there is reported to all of them
+    if (ctx->shape.kvh <= kStaticMaxGroups) {
+        StaticScratch *shared = nullptr;
+        HIP_TRY(ctx, scratch_on_device(ctx->desc.device, &shared));
+        HIP_TRY(ctx, hipMemcpy(sync.data(), shared->sync, sync.size() * sizeof(DecodeGroupSync), hipMemcpyDeviceToHost));
+        for (const DecodeGroupSync &g : sync) {
+            if (g.lost != 0) *flags |= kFlagMergeIncomplete;
+        }
     }
     return GLM_ATTN_OK;
 }

@@ -192,7 +192,7 @@ struct DecodeArgs {
     __half *k_cache;
     __half *v_cache;
     int nsplit;     // workgroups per KV group
-    int tiles_q, tiles_r;  // tiles of 64 cached keys per workgroup: tiles_q, one more in the first tiles_r
+    int tiles_q, tiles_r;  // tiles of 64 cached keys per workgroup: tiles_q, one more in the last tiles_r
     float *part;    // [kvh][nsplit][kDecodePartFloats] split partials as stamped 64-byte lines
     float *out;     // [h d]
     uint32_t *flags;

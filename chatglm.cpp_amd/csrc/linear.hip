@@ -809,7 +809,12 @@ int glm_linear_create(const glm_linear_desc *desc, glm_linear **out_linear) {
         }
     }
     if ((desc->weight_dtype == GLM_LINEAR_F16 || quant) && l->max_rows > 8) {
-        l->lt = lt_device(desc->device);
+        // A borrowed fp16 weight goes to hipBLASLt only if the caller has stated a size that leaves the slack an
+        // owned weight gets: without it a library kernel that fetches ahead of its last tile would read past the
+        // caller's allocation.  (A quantised weight is expanded into the library's own buffer.)
+        const bool slack_known = l->owns_weight || quant ||
+                                 (uint64_t)desc->weight_bytes >= (uint64_t)weight_bytes(*desc) + kOperandSlack;
+        l->lt = slack_known ? lt_device(desc->device) : nullptr;
         if (l->lt && !lt_setup(l)) {
             l->lt = nullptr;
         }

@@ -130,6 +130,12 @@ int glm_attn_forward(glm_attn_ctx *ctx, int32_t layer, const float *qkv, int64_t
 int glm_attn_rope_append(glm_attn_ctx *ctx, int32_t layer, const float *qkv, int64_t qkv_row_stride,
                          const int32_t *position_ids, int32_t qlen, int32_t n_past, void *stream);
 
+/* The second half of forward alone: attention of the queries that the last glm_attn_rope_append of this
+   context left in its scratch (same qlen and n_past) over the cache, masked as forward masks
+   (chatglm.cpp:678-717).  rope_append followed by attend is forward for qlen > 1, launch for launch. */
+int glm_attn_attend(glm_attn_ctx *ctx, int32_t layer, const float *attention_mask, int32_t qlen, int32_t n_past,
+                    float *out, void *stream);
+
 /* forward for qlen == 1 through the fused split-KV kernel: rope, append, attention and the merge of
    the split partials in one launch.  EUNSUPPORTED unless d == 128, h / kvh <= 16 and L % 8 == 0. */
 int glm_attn_decode(glm_attn_ctx *ctx, int32_t layer, const float *qkv, const int32_t *position_ids,

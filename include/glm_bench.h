@@ -1,5 +1,6 @@
 /*
- * Measurement aids of libglm_attn.so for `bench.py --ceiling`.  They have no counterpart in the reference
+ * Measurement aids for `bench.py --ceiling`, in a library of their own (libglm_bench.so; the drop-in library
+ * libglm_attn.so exports none of them).  They have no counterpart in the reference
  * and are no part of the attention path: kernels that only load, shaped like a launch of the decode
  * kernel, so that the read rate this GPU gives such a launch can be measured beside the kernel's own, and
  * loops of matrix instructions, so that what the matrix pipes sustain can be measured beside the prefill kernel.
@@ -27,6 +28,21 @@ enum glm_bench_pattern {
    `sink` is a device float that is never written in practice.  Returns a glm_attn status. */
 int glm_bench_read(int pattern, const void *base, int32_t cache_rows, int32_t kv_heads, size_t bytes, float *sink,
                    void *stream);
+
+enum glm_bench_policy {
+    GLM_BENCH_POLICY_PLAIN = 0,     /* global_load_dwordx4 */
+    GLM_BENCH_POLICY_NT = 1,        /* ... nt: non-temporal, the lines are not kept in the caches */
+    GLM_BENCH_POLICY_SC1 = 2,       /* ... sc1: performed at the device's coherence point */
+    GLM_BENCH_POLICY_SC0_SC1_NT = 3 /* ... sc0 sc1 nt */
+};
+
+/* Launches one read of `bytes` contiguous bytes at `base` (device) with bytes / (waves x loads KiB) workgroups of
+   `waves` waves, every lane `loads` loads of 16 bytes issued up front under the given policy; through_lds != 0:
+   the loads go straight to LDS (global_load_lds_dwordx4; policies PLAIN and NT).  `bytes` must be a multiple of
+   waves x loads KiB.  GLM_ATTN_EUNSUPPORTED for a (waves, loads) pair the library has no kernel for: it has
+   (8,16) (4,16) (4,32) (16,8) (8,8) (4,8) (16,16), through LDS (8,16) (4,16) (4,32). */
+int glm_bench_read_sweep(int policy, int32_t waves, int32_t loads, int32_t through_lds, const void *base, size_t bytes,
+                         float *sink, void *stream);
 
 enum glm_bench_mfma_pattern {
     GLM_BENCH_MFMA_32X32X16 = 0,     /* nothing but v_mfma_f32_32x32x16_f16, two waves per SIMD on every CU */

@@ -23,7 +23,8 @@
  * Calls with more than 8 rows are plain GEMMs (fp16 x fp16, fp32 accumulation and output) on the library's own MFMA
  * kernel after the rows have been rounded.  With GLM_LINEAR_HIPBLASLT=1 in the environment when the layer is created
  * they go to hipBLASLt instead (bias epilogue; the own kernel for shapes it has no algorithm for): faster, but off
- * by default, because two timing programs that drove it ended in GPU memory faults whose cause was never shown.
+ * by default, because two timing programs that drove it ended in GPU memory faults whose cause was never shown; a
+ * caller-owned fp16 weight takes that branch only when weight_bytes states at least 4096 bytes beyond the tensor.
  *
  * All pointers named "device" are HIP device pointers; calls are asynchronous on the given stream.  Status
  * codes are those of glm_attn.h (0 = ok, negative = error; glm_attn_strerror names them).
@@ -60,8 +61,11 @@ typedef struct glm_linear_desc {
     int32_t weight_dtype; /* glm_linear_dtype */
     int32_t use_bias;     /* 0: no bias tensor (the reference's use_bias = false) */
     int32_t max_rows;     /* most input rows of any call; 0 means 1.  Above 8 it sizes the fp16 staging of the input
-                             (max_rows x in_features x 2 bytes), one buffer per device shared by all layers:
-                             calls with more than 8 rows on one device must not overlap on different streams */
+                             (max_rows x in_features x 2 bytes) and, for weights of fewer 128-feature tiles than the
+                             GPU has CUs, the fp32 partial sums of calls cut along the input features (up to
+                             8 x min(max_rows, 128) x out_features x 4 bytes): one buffer of each kind per device,
+                             shared by all layers: calls with more than 8 rows on one device must not overlap on
+                             different streams */
     int32_t device;       /* HIP device ordinal */
     void *weight;         /* optional caller-owned device tensor [out_features][in_features] (quantised types:
                              ggml blocks); NULL: the library allocates (zero-filled) and the caller fills it

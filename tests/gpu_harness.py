@@ -163,6 +163,10 @@ class Pair:
                                   qkv_row_stride=stride)
         elif entry == "rope_append":  # the first half alone: caches only, no output
             st = self.ctx.rope_append(layer, qkv_d.data_ptr(), pos_d.data_ptr(), qlen, n_past, qkv_row_stride=stride)
+        elif entry == "rope_append+attend":  # the two halves of forward as two calls
+            st = self.ctx.rope_append(layer, qkv_d.data_ptr(), pos_d.data_ptr(), qlen, n_past, qkv_row_stride=stride)
+            pkg.check(st, "glm_attn_rope_append")
+            st = self.ctx.attend(layer, qlen, n_past, out_d.data_ptr(), attention_mask_ptr=mp)
         elif entry == "decode":
             st = self.ctx.decode(layer, qkv_d.data_ptr(), n_past, out_d.data_ptr(),
                                  position_ids_ptr=None if host_pos else pos_d.data_ptr(),

@@ -127,16 +127,20 @@ def test_library_exports_every_symbol_of_the_block_header():
     assert lib.glm_block_activation_forward(1, 4, 7, 1, None) == pkg.EINVAL  # no such activation
 
 
-def test_library_exports_every_symbol_of_the_bench_header():
-    lib = pkg.lib()
+def test_bench_library_exports_every_symbol_of_the_bench_header_and_the_drop_in_none():
+    lib = pkg.bench_lib()
     names = declared_symbols("glm_bench.h", "glm_bench_")
-    names = [n for n in names if n != "glm_bench_pattern"]
-    assert names == ["glm_bench_mfma", "glm_bench_read"]
+    names = [n for n in names if n not in ("glm_bench_pattern", "glm_bench_policy", "glm_bench_mfma_pattern")]
+    assert names == ["glm_bench_mfma", "glm_bench_read", "glm_bench_read_sweep"]
     for n in names:
-        assert hasattr(lib, n), f"{n} is declared in include/glm_bench.h but not exported"
+        assert hasattr(lib, n), f"{n} is declared in include/glm_bench.h but not exported by libglm_bench.so"
+        assert not hasattr(pkg.lib(), n), f"{n} is a measurement aid and must not be exported by libglm_attn.so"
     assert sorted(pkg.BENCH_SYMBOLS) == names
     assert lib.glm_bench_read(pkg.BENCH_READ_LINEAR, None, 256, 2, 0, None, None) == pkg.EINVAL
     assert lib.glm_bench_mfma(pkg.BENCH_MFMA_32X32X16, None, 0, 1, None, None, None) == pkg.EINVAL
+    # shapes are checked before anything is launched
+    assert lib.glm_bench_read_sweep(pkg.BENCH_POLICY_NT, 8, 16, 0, None, 1 << 25, None, None) == pkg.EINVAL
+    assert lib.glm_bench_read_sweep(pkg.BENCH_POLICY_NT, 8, 16, 0, 1, 1000, 1, None) == pkg.EINVAL
 
 
 def test_library_exports_every_symbol_of_the_model_file_header():

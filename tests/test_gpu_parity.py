@@ -242,6 +242,27 @@ def test_padded_qkv_rows(H, entry, interleaved, kvh, rope_type):
     p.close()
 
 
+@pytest.mark.parametrize("kw,qlen,n_past", [
+    (dict(kvh=2, max_length=512), 37, 0),       # causal prompt, MFMA kernel
+    (dict(kvh=2, max_length=512), 5, 137),      # unmasked continuation
+    (dict(kvh=32, max_length=512, rope_type="glm1"), 20, 0),  # v1 additive mask
+    (dict(h=4, kvh=2, d=64, max_length=40), 7, 3),            # generic kernel
+])
+def test_rope_append_then_attend_is_forward(H, kw, qlen, n_past):
+    """glm_attn_rope_append followed by glm_attn_attend does what glm_attn_forward does (chatglm.cpp:655-717)."""
+    kw = dict(kw)
+    if kw.get("rope_type") == "glm1":
+        kw.update(rope_type=H.orc.ROPE_CHATGLM, mask_type=H.orc.MASK_CHATGLM)
+    p = H.Pair(**kw)
+    if n_past:
+        p.fill_past(0, n_past, seed=5)
+    qkv = p.random_qkv(qlen, seed=60 + qlen)
+    out, ref, _ = p.forward(0, qkv, n_past, entry="rope_append+attend", n_ctx=300)
+    p.assert_caches_equal(0, "rope_append + attend")
+    H.assert_close(out, ref, f"rope_append + attend, qlen {qlen}")
+    p.close()
+
+
 def test_range_errors(H):
     p = H.Pair(max_length=64)
     import torch
