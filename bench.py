@@ -27,7 +27,20 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
 # HBM bytes one decode_kernel launch of this workload moves, from two rocprofv3 --pmc runs of this script
 # (FETCH_SIZE 17,783 KiB x 2.000, WRITE_SIZE 2,073 KiB x 1.000; scales from a 256 MiB device copy in the same runs)
-DECODE_TRAFFIC_BYTES_PER_LAUNCH = 38_540_000
+DECODE_TRAFFIC_PROFILE = os.path.join("profiles", "decode_kernel_glm4_32k_hbm_traffic_pmc.txt")
+
+
+def decode_traffic_bytes_per_launch():
+    """HBM bytes per decode launch from the committed counter summary (its line `traffic_bytes_per_launch: N`):
+    the figure is refreshed with the profile, not kept as a constant here.  None when the file holds no such line."""
+    import re
+
+    try:
+        text = open(os.path.join(os.path.dirname(os.path.abspath(__file__)), DECODE_TRAFFIC_PROFILE)).read()
+    except OSError:
+        return None
+    m = re.search(r"^traffic_bytes_per_launch:\s*([0-9_,]+)", text, flags=re.M)
+    return int(m.group(1).replace(",", "").replace("_", "")) if m else None
 MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16
 
 H, KVH, D = 32, 2, 128
@@ -382,7 +395,8 @@ def main():
                 "unit": "GB/s",
                 "frac": round(bytes_layer / (ms * 1e-3 / LAYERS) / 1e9 / HBM_PEAK_GBS, 4),
                 "bytes_per_launch": bytes_layer,
-                "traffic": DECODE_TRAFFIC_BYTES_PER_LAUNCH,
+                "traffic": decode_traffic_bytes_per_launch(),
+                "traffic_source": DECODE_TRAFFIC_PROFILE,
             },
         })
 
@@ -473,10 +487,17 @@ def main():
                     torch.cuda.synchronize()
                 return e0.elapsed_time(e1) * 1e3 / (10 * c_layers)  # us per layer
 
+            def c_attend():
+                for l in range(c_layers):
+                    st = ctx2.attend(l, c_q, 0, out_c[l].data_ptr(), stream=sh)
+                    if st != 0:
+                        pkg.check(st, "glm_attn_attend")
+
             us_call, us_rope = c_time(c_forward), c_time(c_rope)
+            us_attend = c_time(c_attend)  # the queries of the last rope_append are still in the context's scratch
             assert bool(torch.isfinite(out_c).all()), "causal prompt produced non-finite output"
             c_flops = 4 * c_h * D * (c_q * (c_q + 1) // 2)
-            us_kernel = us_call - us_rope
+            us_kernel = us_attend
             result["prefill_causal_2048"] = {
                 "workload": "ChatGLM3-6B shape (32 heads, 2 KV groups, max_length 8192): one 2048-token chunk at "
                             "n_past=0, causal, per layer",
@@ -485,7 +506,9 @@ def main():
                 "tokens_per_s": round(c_q / (us_call * 1e-6), 1),
                 "tflops_whole_call": round(c_flops / us_call / 1e6, 1),
                 "roofline": {"bound": "mfma", "kernel": "prefill_kernel",
-                             "duration": "the call minus rope_append_kernel timed alone (both launches of the call)",
+                             "duration": "glm_attn_attend alone (the second launch of the call), events around "
+                                         "back-to-back launches over 4 layers",
+                             "us_per_launch": round(us_attend, 2),
                              "achieved": round(c_flops / us_kernel / 1e6, 1), "peak": MFMA_FP16_PEAK_TFLOPS,
                              "unit": "TFLOP/s", "frac": round(c_flops / us_kernel / 1e6 / MFMA_FP16_PEAK_TFLOPS, 4),
                              "flops_per_launch": c_flops},
@@ -739,6 +762,49 @@ def main():
             "sample": f"single layers of the decode workload for 12 s: {reps} timed passes after 1 warm-up over 8 "
                       f"layers' caches in turn (CPU restatement of the reference graph, {threads} threads of "
                       f"{os.cpu_count()} logical CPUs); us_per_token = 40 x the per-layer time",
+        }
+
+    # ------------------------------------------------------------------ CPU beside the prefill chunk (bounded sample)
+    if not args.skip_cpu and not args.skip_prefill and "prefill" in result:
+        import numpy as np
+
+        sys.path.insert(0, os.path.join(ROOT, "oracle"))
+        import glm_oracle as orc
+
+        qlen, n_past = PREFILL_Q, PREFILL_N_PAST
+        threads = orc.reference_threads(qlen)  # the reference's prompt policy: the physical cores (chatglm.cpp:476-499)
+        ocfg = orc.make_cfg(num_attention_heads=H, num_key_value_heads=KVH, head_size=D, max_length=L,
+                            n_threads=threads)
+        k_ref, v_ref = orc.new_caches(ocfg)
+        k_ref[:, :n_past, :] = orc.randn_f16_bits(3, 1, KVH * n_past * D).reshape(KVH, n_past, D)
+        v_ref[:, :, :n_past] = orc.randn_f16_bits(3, 2, KVH * D * n_past).reshape(KVH, D, n_past)
+        qkv_cpu = orc.randn_f32(3, 0, qlen * width).reshape(qlen, width)
+        pos = orc.position_ids_glm2(qlen, n_past)
+        t0 = time.perf_counter()
+        orc.rope_inplace(ocfg, qkv_cpu, pos)          # rope and append of the whole chunk: timed in full
+        orc.append(ocfg, qkv_cpu, n_past, k_ref, v_ref)
+        t_head = time.perf_counter() - t0
+        block, rows_done = 64, 0
+        out_cpu = np.zeros((qlen, H * D), dtype=np.float32)
+        orc.attend(ocfg, qkv_cpu, n_past, k_ref, v_ref, rows=(qlen - 8, qlen), out=out_cpu)  # warm-up
+        t0 = time.perf_counter()
+        while rows_done < qlen and (rows_done < block or time.perf_counter() - t0 < 12.0):
+            orc.attend(ocfg, qkv_cpu, n_past, k_ref, v_ref, rows=(rows_done, rows_done + block), out=out_cpu)
+            rows_done += block
+        t_rows = time.perf_counter() - t0
+        cpu_layer_s = t_head + t_rows * qlen / rows_done
+        pf_flops = prefill_flops_per_layer(qlen, n_past, causal=False)
+        result["prefill"]["cpu_baseline"] = {
+            "value": round(pf_flops / cpu_layer_s / 1e12, 4),
+            "unit": "TFLOP/s",
+            "tokens_per_s": round(qlen / cpu_layer_s, 1),
+            "s_per_layer": round(cpu_layer_s, 2),
+            "cores": threads,
+            "kind": "port",
+            "sample": f"rope and append of the whole 8192-token chunk ({t_head * 1e3:.0f} ms) plus the attention of "
+                      f"its first {rows_done} token rows against all {n_past + qlen} keys ({t_rows:.1f} s), "
+                      f"extrapolated to 8192 rows (every row costs the same: the chunk is unmasked); CPU restatement "
+                      f"of the reference graph, {threads} threads of {os.cpu_count()} logical CPUs",
         }
 
     ctx.close()

@@ -25,6 +25,15 @@ def test_algorithmic_bytes_and_flops_of_the_headline_configs():
     assert b.prefill_flops_per_layer(2048, 0, causal=True) == 4 * 32 * 128 * (2048 * 2049 // 2)
 
 
+def test_traffic_figure_comes_from_the_committed_counter_summary():
+    b = load_bench()
+    text = open(os.path.join(ROOT, b.DECODE_TRAFFIC_PROFILE)).read()
+    n = b.decode_traffic_bytes_per_launch()
+    assert n is not None and f"traffic_bytes_per_launch: {n:,}" in text
+    # read once plus the exchange of the partials: between the algorithmic bytes and 1.5 times them
+    assert b.decode_bytes_per_layer(32768) <= n < 1.5 * b.decode_bytes_per_layer(32768)
+
+
 def test_more_than_one_gpu_is_refused_with_a_message():
     r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
     assert r.returncode == 2
