@@ -310,8 +310,9 @@ def test_decode_repeated_launches_reuse_the_handover_state(H):
     p.close()
 
 
-# The merge across workgroups changes shape with the number of splits (split lanes per line 1..16, 1, 2, 4 or 8
-# lines per lane, one wave per quad or all four on one, one or two passes) and with the group size (padding heads).
+# The merge across workgroups changes shape with the number of splits (split lanes per line 1..16; 1, 2, 4 or 8
+# lines per lane and block, up to four quads per block, 16 lines per lane as two blocks) and with the group size
+# (padding heads).
 @pytest.mark.parametrize("h,kvh,max_length,n_past", [
     (32, 2, 8192, 100),    # 2 tiles: one workgroup per group, no exchange
     (32, 2, 8192, 200),    # 4 tiles: the same, a full round
@@ -321,13 +322,13 @@ def test_decode_repeated_launches_reuse_the_handover_state(H):
     (32, 2, 8192, 500),    # 8
     (32, 2, 8192, 1000),   # 16
     (32, 2, 8192, 1500),   # 24
-    (32, 2, 8192, 3000),   # 47: two waves per quad
+    (32, 2, 8192, 3000),   # 47: three lines per lane, code for four
     (32, 2, 8192, 4095),   # 64
-    (32, 2, 8192, 5000),   # 79: four waves per quad
+    (32, 2, 8192, 5000),   # 79: five lines per lane, code for eight
     (32, 2, 8192, 8191),   # 128
     (32, 32, 2048, 1000),  # one head per group, 8 splits
     (8, 2, 4096, 3000),    # four heads per group
-    (16, 1, 16384, 16383), # 256 splits: two batches per lane
+    (16, 1, 16384, 16383), # 256 splits: 16 lines per lane, two blocks of eight
 ])
 def test_decode_merge_geometries(H, h, kvh, max_length, n_past):
     p = H.Pair(h=h, kvh=kvh, max_length=max_length, cache_fill=0x7E00)

@@ -52,6 +52,28 @@ def test_contexts_of_different_shapes_take_turns(H):
     q.close()
 
 
+@pytest.mark.parametrize("kw,n_past", [
+    (dict(max_length=8192), 700),            # 11 splits of one tile, 12 quads a slice
+    (dict(max_length=8192), 8191),           # 128 splits, one quad a slice
+    (dict(h=8, kvh=8, max_length=2048), 1500),  # one head per group: grouped stamps of 8 groups side by side
+    (dict(h=8, kvh=2, max_length=4096), 3000),  # four heads per group
+])
+def test_static_slow_path_when_workgroups_do_not_wait(H, kw, n_past):
+    """The give-up / redo path of the exchange (wait bound 0: every wave gives up on its first look, flags its slice,
+    and the workgroups that finish later redo what is still missing) on the static array: grouped stamps, the shared
+    claim words.  Every kernel exits normally; the result must not change and nothing may be reported lost."""
+    p = H.Pair(**kw)
+    p.ctx.set_spin_limit_us(0)
+    for rep in range(3):
+        qkv = p.random_qkv(1, seed=700 + rep)
+        p.fill_past(0, n_past, seed=n_past)
+        out, ref, _ = p.forward(0, qkv, n_past, host_pos=True, entry="decode_static")
+        p.assert_caches_equal(0, "static slow path")
+        H.assert_close(out, ref, f"static slow path rep {rep}")
+    assert p.ctx.device_flags() == 0  # the static array's own count of lost slices is part of the flags
+    p.close()
+
+
 def test_more_groups_than_the_array_has_room_for(H):
     import torch
 
