@@ -372,10 +372,10 @@ __device__ inline int poll_block(const MergeGeom &mg, const int (&q)[PC], const 
 #pragma unroll
         for (int k = 0; k < NLP; k++) {
             const int i = pp * NLP + k;
-            const int sp = ((k0 + k) << mg.sl_log) + s;
+            const int sp = merge_split_of(k0 + k, mg.sl_log, s);
             r[i] = uintx4{0u, 0u, 0u, 0u};
             need[i] = qvalid[pp] && sp < mg.nsplit;
-            p[i] = mg.part_g + ((int64_t)q[pp] * mg.nsplit + (sp < mg.nsplit ? sp : 0)) * 16 + piece * 4;
+            p[i] = mg.part_g + merge_piece_offset(q[pp], mg.nsplit, sp < mg.nsplit ? sp : 0, piece);
             pending[i] = __ballot(need[i]);
         }
     }
@@ -459,14 +459,15 @@ template <int NLP, int PC>
 __device__ inline int merge_passes(const MergeGeom &mg, int q_begin, int q_end, int wi, int nw, int lane,
                                    unsigned long long t0, unsigned long long limit) {
     const int qw = 16 >> mg.sl_log;
-    const int piece = lane & 3, qslot = (lane >> 2) & (qw - 1), s = lane >> (6 - mg.sl_log);
+    int piece, qslot, s;
+    merge_lane(mg.sl_log, lane, &piece, &qslot, &s);
     for (int q0 = q_begin + wi * qw; q0 < q_end; q0 += PC * nw * qw) {
         int q[PC];
         bool qvalid[PC];
         Fold acc[PC];
 #pragma unroll
         for (int pp = 0; pp < PC; pp++) {
-            const int qq = q0 + pp * nw * qw + qslot;
+            const int qq = merge_quad_of(q0, pp, nw, mg.sl_log, qslot);
             qvalid[pp] = qq < q_end;
             q[pp] = qvalid[pp] ? qq : q_end - 1;
         }
@@ -502,6 +503,8 @@ __device__ inline int merge_quads(const MergeGeom &mg, int q_begin, int q_end, i
                                   unsigned long long t0, unsigned long long limit, bool bump) {
     // the code that runs is the one for the number of lines a lane really has: at 2.3 ns a vector instruction,
     // folding lines that are not there costs as much as folding lines that are
+    // (the template arguments are merge_shape's nlp and pc, spelled as ranges of nl: within an instantiation the
+    // compiler then knows how many blocks of lines there are)
     const int failed = mg.nl <= 1   ? merge_passes<1, 4>(mg, q_begin, q_end, wi, nw, lane, t0, limit)
                        : mg.nl <= 2 ? merge_passes<2, 2>(mg, q_begin, q_end, wi, nw, lane, t0, limit)
                        : mg.nl <= 4 ? merge_passes<4, 1>(mg, q_begin, q_end, wi, nw, lane, t0, limit)
@@ -923,13 +926,11 @@ __device__ inline void decode_body(const DecodeArgs &a, DecodeShared &sh) {
     DecodeGroupSync *sy = nullptr;
     unsigned long long *claim = nullptr;
     auto resolve = [&]() {
-        qps = (total_quads + a.nsplit - 1) / a.nsplit;
+        qps = merge_quads_per_slice(total_quads, a.nsplit);
         mg.nsplit = a.nsplit;
-        mg.sl_log = 0;
-        while (mg.sl_log < 4 && (1 << mg.sl_log) < a.nsplit) {
-            mg.sl_log++;
-        }
-        mg.nl = (a.nsplit + (1 << mg.sl_log) - 1) >> mg.sl_log;
+        const MergeShape ms = merge_shape(a.nsplit);
+        mg.sl_log = ms.sl_log;
+        mg.nl = ms.nl;
         mg.part_g = a.part + (int64_t)g * a.nsplit * kDecodePartFloats;
         mg.out_g = a.out + (int64_t)g * G * D;
         mg.gen_word = &a.sync[g].gen;

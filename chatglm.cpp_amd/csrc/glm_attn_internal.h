@@ -86,6 +86,45 @@ __host__ __device__ inline void decode_tile_range(int nsplit, int tiles_q, int t
     *te = *tb + tiles_q + (split >= extra_from ? 1 : 0);
 }
 
+// decode_kernel, the fold of the split partials.  The partials of a KV group are lines of 64 bytes, one per
+// (head, 16 output dims) = "quad" q = head * 8 + quad and split, laid out [q][split][16 floats]; a line is four
+// 16-byte pieces.  The quads are dealt out in slices of qps to the group's workgroups, a slice's quads to the waves
+// that fold (wave wi of nw).  Lane (s, quad slot, piece) of a wave takes piece `piece` of the lines of splits
+// s, s + SL, ... (SL = 1 << sl_log, nl lines) of the quad in its slot; a wave loads the lines of pc passes of its
+// 16 / SL quad slots, nlp lines each, in one block (nl > nlp: further blocks of nlp lines).
+struct MergeShape {
+    int sl_log, nl;  // split lanes per (quad, piece): 1 << sl_log; lines per lane and quad
+    int nlp, pc;     // lines per lane, quad and block (1, 2, 4, 8); quads per lane and block (4, 2, 1, 1)
+};
+__host__ __device__ inline MergeShape merge_shape(int nsplit) {
+    MergeShape m;
+    m.sl_log = 0;
+    while (m.sl_log < 4 && (1 << m.sl_log) < nsplit) {
+        m.sl_log++;
+    }
+    m.nl = (nsplit + (1 << m.sl_log) - 1) >> m.sl_log;
+    m.nlp = m.nl <= 1 ? 1 : m.nl <= 2 ? 2 : m.nl <= 4 ? 4 : 8;
+    m.pc = m.nlp == 1 ? 4 : m.nlp == 2 ? 2 : 1;
+    return m;
+}
+__host__ __device__ inline int merge_quads_per_slice(int total_quads, int nsplit) {
+    return (total_quads + nsplit - 1) / nsplit;
+}
+__host__ __device__ inline void merge_lane(int sl_log, int lane, int *piece, int *qslot, int *s) {
+    *piece = lane & 3;
+    *qslot = (lane >> 2) & ((16 >> sl_log) - 1);
+    *s = lane >> (6 - sl_log);  // in the upper bits of the lane index, where reductions are cheap
+}
+// the quad of pass pp of the block that starts at q0 (q0 = q_begin + wi * qw, then + pc * nw * qw per block)
+__host__ __device__ inline int merge_quad_of(int q0, int pp, int nw, int sl_log, int qslot) {
+    return q0 + pp * nw * (16 >> sl_log) + qslot;
+}
+__host__ __device__ inline int merge_split_of(int k, int sl_log, int s) { return (k << sl_log) + s; }
+// where piece `piece` of the line of (quad q, split sp) starts, in floats from the group's first line
+__host__ __device__ inline int64_t merge_piece_offset(int q, int nsplit, int sp, int piece) {
+    return ((int64_t)q * nsplit + sp) * 16 + piece * 4;
+}
+
 // prefill_kernel: rows of 128 per item, items of one unit (a head, or a KV group when a few tokens are packed with
 // the heads of their group), four-wave or eight-wave workgroups, and the cut along the keys with its partials.
 constexpr int kPrefillRows = 128;        // rows (tokens) per workgroup

@@ -63,6 +63,75 @@ static int check_decode() {
     return 0;
 }
 
+// The fold of the split partials (merge_shape, merge_lane, merge_quad_of, merge_split_of, merge_piece_offset: what the
+// score waves of decode_kernel use): for every split count and group size, walked the way the kernel walks it
+// (slices of quads per workgroup, waves of a workgroup, blocks of passes, blocks of lines, 64 lanes), every piece
+// of every line of every quad of the group is taken exactly once, by a lane that also writes that quad's output
+// piece or has a lane beside it that does, and lies inside the lines the group's workgroups have written.
+static int check_decode_merge() {
+    char what[160];
+    for (int G : {1, 2, 4, 16}) {
+        for (int nsplit = 2; nsplit <= kDecodeMaxSplits; nsplit += (nsplit < 140 ? 1 : 31)) {
+            for (int nw : {4, 1}) {  // the score waves of a workgroup, or one wave redoing a slice on its own
+                const int total_quads = G * (kFastHeadSize / 16);
+                const MergeShape ms = merge_shape(nsplit);
+                const int qps = merge_quads_per_slice(total_quads, nsplit);
+                const int SL = 1 << ms.sl_log, qw = 16 >> ms.sl_log;
+                snprintf(what, sizeof(what), "merge G %d nsplit %d nw %d: sl_log %d nl %d nlp %d pc %d qps %d", G, nsplit, nw,
+                         ms.sl_log, ms.nl, ms.nlp, ms.pc, qps);
+                CHECK(SL * ms.nl >= nsplit && SL * (ms.nl - 1) < nsplit);  // the split lanes cover the splits, no line idle
+                CHECK(ms.nlp >= 1 && ms.nlp <= 8 && ms.nlp * ms.pc <= 8);  // loads per lane and block: ld_lines has 1, 2, 4, 8
+                CHECK(ms.nl <= ms.nlp || ms.nlp == 8);                      // only blocks of 8 lines repeat
+                CHECK(qps >= 1 && (int64_t)qps * nsplit >= total_quads);
+                const int64_t group_floats = (int64_t)nsplit * kDecodePartFloats;  // what the group's workgroups write
+                std::vector<int> taken((size_t)total_quads * nsplit * 4, 0), written((size_t)total_quads * 4, 0);
+                for (int split = 0; split < nsplit; split++) {
+                    const int q_begin = split * qps;
+                    const int q_end = (split + 1) * qps < total_quads ? (split + 1) * qps : total_quads;
+                    for (int wi = 0; wi < nw; wi++) {
+                        for (int q0 = q_begin + wi * qw; q0 < q_end; q0 += ms.pc * nw * qw) {
+                            for (int k0 = 0; k0 < ms.nl; k0 += ms.nlp) {
+                                for (int lane = 0; lane < 64; lane++) {
+                                    int piece, qslot, sl;
+                                    merge_lane(ms.sl_log, lane, &piece, &qslot, &sl);
+                                    CHECK(piece >= 0 && piece < 4 && qslot >= 0 && qslot < qw && sl >= 0 && sl < SL);
+                                    for (int pp = 0; pp < ms.pc; pp++) {
+                                        const int q = merge_quad_of(q0, pp, nw, ms.sl_log, qslot);
+                                        if (q >= q_end) continue;  // qvalid
+                                        if (k0 == 0 && sl == 0) written[(size_t)q * 4 + piece]++;
+                                        for (int k = 0; k < ms.nlp; k++) {
+                                            const int sp = merge_split_of(k0 + k, ms.sl_log, sl);
+                                            if (sp >= nsplit) continue;  // need
+                                            const int64_t off = merge_piece_offset(q, nsplit, sp, piece);
+                                            CHECK(off >= 0 && off + 4 <= group_floats);
+                                            CHECK(off == ((int64_t)q * nsplit + sp) * 16 + piece * 4);
+                                            taken[((size_t)q * nsplit + sp) * 4 + piece]++;
+                                        }
+                                    }
+                                }
+                            }
+                        }
+                    }
+                }
+                for (size_t i = 0; i < taken.size(); i++) CHECK(taken[i] == 1);
+                for (size_t i = 0; i < written.size(); i++) CHECK(written[i] == 1);
+                // the writer's side: lane (j, c) of output wave w stores piece c of quads 2 w, 2 w + 1 of head j
+                for (int split = 0; split < nsplit; split += (nsplit > 8 ? nsplit - 1 : 1)) {
+                    for (int j = 0; j < G; j++) {
+                        for (int quad = 0; quad < 8; quad++) {
+                            for (int c = 0; c < 4; c++) {
+                                const int64_t off = (int64_t)(j * 8 + quad) * nsplit * 16 + split * 16 + c * 4;
+                                CHECK(off == merge_piece_offset(j * 8 + quad, nsplit, split, c) && off + 4 <= group_floats);
+                            }
+                        }
+                    }
+                }
+            }
+        }
+    }
+    return 0;
+}
+
 static int check_prefill() {
     char what[200];
     const int D = kFastHeadSize;
@@ -153,7 +222,7 @@ static int check_splitk() {
 }
 
 int main() {
-    if (check_decode() || check_prefill() || check_splitk()) return 1;
+    if (check_decode() || check_decode_merge() || check_prefill() || check_splitk()) return 1;
     printf("ok\n");
     return 0;
 }
