@@ -18,7 +18,7 @@ MASK_RULE_REFERENCE, MASK_RULE_CAUSAL_OFFSET = 0, 1
 
 # every symbol include/glm_attn.h declares
 SYMBOLS = [
-    "glm_attn_default_desc", "glm_attn_kv_bytes", "glm_attn_create", "glm_attn_destroy", "glm_attn_cache_ptrs",
+    "glm_attn_default_desc", "glm_attn_kv_bytes", "glm_attn_create", "glm_attn_destroy", "glm_attn_set_qkv_views", "glm_attn_cache_ptrs",
     "glm_attn_forward", "glm_attn_rope_append", "glm_attn_attend", "glm_attn_decode", "glm_attn_decode_static", "glm_attn_prefill",
     "glm_attn_load_prefix_cache", "glm_attn_position_ids_glm2", "glm_attn_position_ids_glm",
     "glm_attn_attention_mask_glm", "glm_attn_scale_add", "glm_attn_device_flags", "glm_attn_set_spin_limit_us", "glm_attn_last_hip_error", "glm_attn_strerror",
@@ -251,6 +251,8 @@ def lib():
     L.glm_attn_create.restype = c.c_int
     L.glm_attn_destroy.argtypes = [P]
     L.glm_attn_destroy.restype = None
+    L.glm_attn_set_qkv_views.argtypes = [P, c.c_int64, c.c_int64, c.c_int64, c.c_int64]
+    L.glm_attn_set_qkv_views.restype = c.c_int
     L.glm_attn_cache_ptrs.argtypes = [P, c.c_int32, c.POINTER(P), c.POINTER(P)]
     L.glm_attn_cache_ptrs.restype = c.c_int
     L.glm_attn_forward.argtypes = [P, c.c_int32, P, c.c_int64, P, P, P, c.c_int32, c.c_int32, P, P]
@@ -395,6 +397,9 @@ class Context:
         return lib().glm_attn_forward(self.handle, layer, qkv_ptr, qkv_row_stride, attention_mask_ptr,
                                       position_ids_ptr, ctypes.cast(hp, ctypes.c_void_p) if hp is not None else None,
                                       qlen, n_past, out_ptr, stream)
+
+    def set_qkv_views(self, q_offset, k_offset, v_offset, head_stride):
+        return lib().glm_attn_set_qkv_views(self.handle, q_offset, k_offset, v_offset, head_stride)
 
     def rope_append(self, layer, qkv_ptr, position_ids_ptr, qlen, n_past, qkv_row_stride=0, stream=None):
         return lib().glm_attn_rope_append(self.handle, layer, qkv_ptr, qkv_row_stride, position_ids_ptr, qlen, n_past,

@@ -16,6 +16,8 @@ struct glm_attn_ctx {
     glm_attn_desc desc;
     Shape shape;
     QkvLayout layout;  // row_stride filled per call
+    int64_t row_extent;  // floats of a row that the three views reach: the default row stride
+    bool views_aligned;  // offsets and head stride are multiples of 4 floats: the 16-byte loads of the decode kernel
     RopeSpec rope;
     float scale;
     int max_qlen;
@@ -176,9 +178,16 @@ int check_call(const glm_attn_ctx *c, int layer, int qlen, int n_past) {
 
 QkvLayout call_layout(const glm_attn_ctx *c, int64_t row_stride) {
     QkvLayout l = c->layout;
-    const int64_t width = (int64_t)(c->shape.h + 2 * c->shape.kvh) * c->shape.d;
-    l.row_stride = row_stride > 0 ? row_stride : width;
+    l.row_stride = row_stride > 0 ? row_stride : c->row_extent;
     return l;
+}
+
+// One past the last float of a row that the views (offsets, head stride) reach.
+int64_t views_extent(const Shape &s, int64_t q_off, int64_t k_off, int64_t v_off, int64_t head_stride) {
+    const int64_t q_end = q_off + (int64_t)(s.h - 1) * head_stride + s.d;
+    const int64_t k_end = k_off + (int64_t)(s.kvh - 1) * head_stride + s.d;
+    const int64_t v_end = v_off + (int64_t)(s.kvh - 1) * head_stride + s.d;
+    return q_end > k_end ? (q_end > v_end ? q_end : v_end) : (k_end > v_end ? k_end : v_end);
 }
 
 // Which keys a call masks: (causal flag, additive mask pointer).  chatglm.cpp:689-707.
@@ -216,6 +225,7 @@ int stage_positions(glm_attn_ctx *c, const int32_t *position_ids, const int32_t 
 
 int do_rope_append(glm_attn_ctx *c, int layer, const float *qkv, int64_t row_stride, const int32_t *dev_pos, int qlen,
                    int n_past, hipStream_t stream) {
+    if (row_stride > 0 && row_stride < c->row_extent) return GLM_ATTN_EINVAL;  // rows would run into each other
     RopeAppendArgs ra;
     ra.qkv = qkv;
     ra.lay = call_layout(c, row_stride);
@@ -358,6 +368,8 @@ int glm_attn_create(const glm_attn_desc *desc, glm_attn_ctx **out_ctx) {
         c->layout.k_off = s.h * s.d;
         c->layout.v_off = (s.h + s.kvh) * s.d;
     }
+    c->row_extent = views_extent(s, c->layout.q_off, c->layout.k_off, c->layout.v_off, c->layout.head_stride);
+    c->views_aligned = ((c->layout.q_off | c->layout.k_off | c->layout.v_off | c->layout.head_stride) & 3) == 0;
     c->fast = (s.d == kFastHeadSize) && (s.G <= kMaxGroupHeads) && (s.L % 8 == 0);
     c->layer_halfs = 2u * (size_t)s.kvh * (size_t)s.L * (size_t)s.d;
 
@@ -470,6 +482,22 @@ void glm_attn_destroy(glm_attn_ctx *ctx) {
     free_ctx(ctx);
 }
 
+int glm_attn_set_qkv_views(glm_attn_ctx *ctx, int64_t q_offset, int64_t k_offset, int64_t v_offset,
+                           int64_t head_stride) {
+    if (!ctx) return GLM_ATTN_EINVAL;
+    const Shape &s = ctx->shape;
+    if (q_offset < 0 || k_offset < 0 || v_offset < 0 || head_stride < s.d) return GLM_ATTN_EINVAL;
+    const int64_t extent = views_extent(s, q_offset, k_offset, v_offset, head_stride);
+    if (extent > 0x7fffffff) return GLM_ATTN_ERANGE;  // the kernels keep the offsets in 32 bits
+    ctx->layout.q_off = (int)q_offset;
+    ctx->layout.k_off = (int)k_offset;
+    ctx->layout.v_off = (int)v_offset;
+    ctx->layout.head_stride = (int)head_stride;
+    ctx->row_extent = extent;
+    ctx->views_aligned = ((q_offset | k_offset | v_offset | head_stride) & 3) == 0;
+    return GLM_ATTN_OK;
+}
+
 int glm_attn_cache_ptrs(const glm_attn_ctx *ctx, int32_t layer, void **k_cache, void **v_cache) {
     if (!ctx) return GLM_ATTN_EINVAL;
     if (layer < 0 || layer >= ctx->desc.num_layers) return GLM_ATTN_ERANGE;
@@ -492,7 +520,7 @@ int glm_attn_decode(glm_attn_ctx *ctx, int32_t layer, const float *qkv, const in
     int rc = check_call(ctx, layer, 1, n_past);
     if (rc != GLM_ATTN_OK) return rc;
     if (!qkv || !out) return GLM_ATTN_EINVAL;
-    if (!ctx->fast || !aligned16(qkv)) return GLM_ATTN_EUNSUPPORTED;
+    if (!ctx->fast || !aligned16(qkv) || !ctx->views_aligned) return GLM_ATTN_EUNSUPPORTED;
     DeviceGuard guard(ctx->desc.device);
     return do_decode(ctx, layer, qkv, position_ids, position_ids_host, n_past, out, (hipStream_t)stream);
 }
@@ -502,7 +530,7 @@ int glm_attn_decode_static(glm_attn_ctx *ctx, int32_t layer, const float *qkv, c
     int rc = check_call(ctx, layer, 1, n_past);
     if (rc != GLM_ATTN_OK) return rc;
     if (!qkv || !out) return GLM_ATTN_EINVAL;
-    if (!ctx->fast || !aligned16(qkv)) return GLM_ATTN_EUNSUPPORTED;
+    if (!ctx->fast || !aligned16(qkv) || !ctx->views_aligned) return GLM_ATTN_EUNSUPPORTED;
     if (ctx->shape.kvh > kStaticMaxGroups) return GLM_ATTN_ESTATIC;
     DeviceGuard guard(ctx->desc.device);
     StaticScratch *shared;
@@ -564,7 +592,7 @@ int glm_attn_forward(glm_attn_ctx *ctx, int32_t layer, const float *qkv, int64_t
     hipStream_t st = (hipStream_t)stream;
 
     // one token, nothing to mask: the fused split-KV kernel
-    if (qlen == 1 && ctx->fast && !mask && aligned16(qkv)) {
+    if (qlen == 1 && ctx->fast && !mask && aligned16(qkv) && ctx->views_aligned) {
         return do_decode(ctx, layer, qkv, position_ids, position_ids_host, n_past, out, st);
     }
     const int32_t *dev_pos;

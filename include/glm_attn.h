@@ -97,6 +97,17 @@ int glm_attn_create(const glm_attn_desc *desc, glm_attn_ctx **out_ctx);
 /* Frees everything the context owns (not a caller-owned kv_buffer).  Synchronises the device. */
 void glm_attn_destroy(glm_attn_ctx *ctx);
 
+/* The three views of the fused projection in their general form (chatglm.cpp:636-653: ggml_view_3d with a byte
+   offset, nb[1] between heads and nb[2] between tokens): q head i of a token starts q_offset + i * head_stride
+   floats into the token's row, k and v heads likewise from k_offset and v_offset; the stride between tokens stays
+   the qkv_row_stride of each call (0 there = the smallest stride that holds all three views).  glm_attn_create
+   sets the two layouts the reference builds (plain: offsets 0, h d, (h + kvh) d, stride d; interleaved_qkv:
+   0, d, 2 d, stride 3 d); this call replaces them for every later call of the context.  head_stride >= d.
+   When an offset or the stride is not a multiple of 4 floats, one-token calls take the two-launch path
+   (glm_attn_decode returns GLM_ATTN_EUNSUPPORTED). */
+int glm_attn_set_qkv_views(glm_attn_ctx *ctx, int64_t q_offset, int64_t k_offset, int64_t v_offset,
+                           int64_t head_stride);
+
 /* Device pointers of one layer's caches: k_cache fp16 [kvh][L][d], v_cache fp16 [kvh][d][L]
    (the public members BasicAttention::k_cache / v_cache, chatglm.h:470-471). */
 int glm_attn_cache_ptrs(const glm_attn_ctx *ctx, int32_t layer, void **k_cache, void **v_cache);

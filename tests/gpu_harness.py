@@ -59,6 +59,7 @@ class Pair:
         self.torch = torch
         self.dev = torch.device(device)
         self.h, self.kvh, self.d, self.nvt = h, kvh, d, nvt
+        self.interleaved = bool(interleaved)
         self.L = max_length + nvt
         self.num_layers = num_layers
         self.rope_type = rope_type
@@ -126,9 +127,12 @@ class Pair:
 
     # ---- one call through both implementations
     def forward(self, layer, qkv, n_past, pos=None, mask=None, host_pos=False, entry="forward", n_ctx=None,
-                oracle_rows=None, use_default_mask=True, row_pad=0):
+                oracle_rows=None, use_default_mask=True, row_pad=0, views=None, default_row_stride=False):
         """row_pad > 0: the device copy of qkv gets that many floats of NaN behind every row and the call is
-        made with qkv_row_stride = width + row_pad (entries "forward", "prefill" and "rope_append")."""
+        made with qkv_row_stride = width + row_pad (entries "forward", "prefill" and "rope_append").
+        views = (q_offset, k_offset, v_offset, head_stride, row_stride): the context has been given these views
+        (set_qkv_views); the device copy of qkv is laid out accordingly, NaN wherever no view reaches;
+        default_row_stride: the call passes qkv_row_stride = 0 (the views' own extent) instead of row_stride."""
         torch = self.torch
         qlen = qkv.shape[0]
         if pos is None:
@@ -145,7 +149,23 @@ class Pair:
             ref = orc.attend(self.ocfg, qkv_ref, n_past, self.ref_k[layer], self.ref_v[layer], attention_mask=mask,
                              rows=oracle_rows)
         stride = 0
-        if row_pad:
+        if views is not None:
+            q_off, k_off, v_off, hs, stride = views
+            laid = np.full((qlen, stride), np.nan, dtype=np.float32)
+            std = qkv.reshape(qlen, -1)
+            d = self.d
+            if self.interleaved:  # the oracle's row is [h][3][d]
+                src = lambda which, i: std[:, (3 * i + which) * d:(3 * i + which + 1) * d]
+            else:
+                base = (0, self.h * d, (self.h + self.kvh) * d)
+                src = lambda which, i: std[:, base[which] + i * d:base[which] + (i + 1) * d]
+            for which, off, n in ((0, q_off, self.h), (1, k_off, self.kvh), (2, v_off, self.kvh)):
+                for i in range(n):
+                    laid[:, off + i * hs:off + i * hs + d] = src(which, i)
+            qkv_d = torch.from_numpy(laid).to(self.dev)
+            if default_row_stride:
+                stride = 0
+        elif row_pad:
             padded = np.full((qlen, self.width + row_pad), np.nan, dtype=np.float32)
             padded[:, :self.width] = qkv
             qkv_d = torch.from_numpy(padded).to(self.dev)
