@@ -52,6 +52,18 @@ def test_contexts_of_different_shapes_take_turns(H):
     q.close()
 
 
+def test_more_groups_than_the_array_has_room_for(H):
+    import torch
+
+    p = H.Pair(h=64, kvh=64, max_length=256)
+    qkv_d = torch.zeros(p.width, device=p.dev)
+    out_d = torch.zeros(p.h * p.d, device=p.dev)
+    st = p.ctx.decode_static(0, qkv_d.data_ptr(), 10, out_d.data_ptr(), position_ids_host=[10])
+    assert st == H.pkg.ESTATIC
+    assert "32" in H.pkg.strerror(st)
+    p.close()
+
+
 @pytest.mark.parametrize("kw,n_past", [
     (dict(max_length=8192), 700),            # 11 splits of one tile, 12 quads a slice
     (dict(max_length=8192), 8191),           # 128 splits, one quad a slice
@@ -71,16 +83,4 @@ def test_static_slow_path_when_workgroups_do_not_wait(H, kw, n_past):
         p.assert_caches_equal(0, "static slow path")
         H.assert_close(out, ref, f"static slow path rep {rep}")
     assert p.ctx.device_flags() == 0  # the static array's own count of lost slices is part of the flags
-    p.close()
-
-
-def test_more_groups_than_the_array_has_room_for(H):
-    import torch
-
-    p = H.Pair(h=64, kvh=64, max_length=256)
-    qkv_d = torch.zeros(p.width, device=p.dev)
-    out_d = torch.zeros(p.h * p.d, device=p.dev)
-    st = p.ctx.decode_static(0, qkv_d.data_ptr(), 10, out_d.data_ptr(), position_ids_host=[10])
-    assert st == H.pkg.ESTATIC
-    assert "32" in H.pkg.strerror(st)
     p.close()
