@@ -1,7 +1,7 @@
-"""Entry points added after the last GPU run of this repository: glm_attn_attend (the second half of forward as a
-call of its own) and glm_attn_set_qkv_views (the three views of the fused projection in their general form,
-chatglm.cpp:636-653), against the oracle through the C-ABI.  Collected late on purpose: these tests have not run on
-a GPU yet, and `pytest -x` should not let a failure here hide the tests of the established path."""
+"""glm_attn_attend (the second half of forward as a call of its own) and glm_attn_set_qkv_views (the three views of
+the fused projection in their general form, chatglm.cpp:636-653), against the oracle through the C-ABI.  The file
+name makes pytest collect these after the tests of forward / decode / prefill themselves: with `pytest -x` a
+failure in a newer entry point then does not hide the tests of the path every caller uses."""
 import pytest
 
 pytestmark = pytest.mark.gpu
